@@ -156,8 +156,8 @@ int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg
 int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                    int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                    int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
-                   int num_pages, float scale, int window, int chunk, int key_chunk, int dtype, int max_context, int single_from,
-                   void *workspace, size_t workspace_bytes, hipStream_t stream);
+                   int num_pages, float scale, int window, int chunk, int key_chunk, const float *sinks, int dtype, int max_context,
+                   int single_from, void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 // The same attention with a bias on every score that depends on the distance alone: score(row, key) = q . k * scale +
 // head_slopes[head] * (key position - row position), float32 `head_slopes[heads]` (for position encodings that bias
@@ -301,7 +301,9 @@ size_t fllm_talking_attention_workspace(int rows, int num_segs, int heads, int v
 // A branch that is normed on its way into the float32 residual stream: v = the sum of the row's `parts` partial branches
 // (branch: [rows, parts, width] of `branch_dtype`), x[r] += v * rsqrt(mean(v^2) + eps) * gain (normalize 0: x[r] += v * gain).
 // With next_w, next_out[r] = rmsnorm(x[r]) * next_w with next_eps (of `next_dtype`) as well.
-int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts, const float *gain, float eps, int normalize,
+// part_weights (float32 [rows * parts], or null): partial row k of a token is multiplied by its weight as it is summed.
+int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts, const float *part_weights, const float *gain, float eps,
+                      int normalize,
                       const float *next_w, float next_eps, void *next_out, int next_dtype, int rows, int width, hipStream_t stream);
 
 // Routed experts, plain kernels.  fllm_route_topk: score = sigmoid(w_router h) in float32 ([E, K] beside rows [rows, K] of
@@ -309,8 +311,10 @@ int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts,
 // among equals) and that score.  fllm_experts_gate_up: for every (row, pick) pair, act[pair] = a(g) * (u + up_offset) with
 // g, u = the gate and up rows of the picked expert times (h[row] * weight), clamped as in fllm_glu_clamped;
 // w_gate_up = [E][2 inter][K].  fllm_experts_down: out[pair] = w_down[e] act[pair], float32; w_down = [E][N][inter].
+// score_mode 1: the score is the softmax of the logits over all experts; renormalize: the picks' weights are divided by their
+// sum (+ 1e-20); route_scale multiplies them.
 int fllm_route_topk(const void *h, int ldh, const void *w_router, int rows, int K, int E, int top, int32_t *ids, float *weights,
-                    int dtype, hipStream_t stream);
+                    int score_mode, int renormalize, float route_scale, int dtype, hipStream_t stream);
 int fllm_experts_gate_up(const void *h, int ldh, const int32_t *ids, const float *weights, int rows, int top, const void *w_gate_up,
                          int E, int inter, int K, void *act, float limit, float alpha, float up_offset, int dtype, hipStream_t stream);
 int fllm_experts_down(const void *act, const int32_t *ids, int pairs, const void *w_down, int E, int N, int inter, float *out, int dtype,
@@ -324,6 +328,40 @@ size_t fllm_experts_grouped_plane_floats(int pairs, int E, int N, int inter);   
 int fllm_experts_grouped(const void *h, int ldh, const int32_t *ids, const float *weights, int rows, int top, const void *w_gate_up,
                          const void *w_down, int E, int inter, int K, int N, void *act, void *xs, float *out, int32_t *work,
                          float *planes, float limit, float alpha, float up_offset, hipStream_t stream);
+
+// ---- mechanisms that carry something from token to token outside the pages (sequence_ops.hip) --------------------------------
+// Rows, segments and slots as in fllm_attention: rows of a segment are consecutive, seg_start[s] is its first row, slots[s] the
+// state slot of its request; rows with row_seg < 0 are padding (outputs zero, no state touched).  A segment's rows continue
+// the state that the request's slot holds.
+// fllm_short_conv: out[t] = x[t] + sum_j w[c][j] x[t - taps + 1 + j] on every channel c (w float32 [width][taps]); the inputs
+// before a step's first row come from state [slots][taps - 1][width] (of `dtype`, zeros at a sequence's start), which
+// afterwards holds the last taps - 1 inputs of the sequence.
+int fllm_short_conv(const void *x, const float *w, void *state, const int32_t *row_seg, const int32_t *seg_start,
+                    const int32_t *slots, int num_segs, void *out, int rows, int width, int taps, int dtype, hipStream_t stream);
+// The same behind a norm with one weight vector, for steps of one row a segment: h = x * rsqrt(mean x^2 + eps) * norm_w is
+// computed from the float32 stream x, convolved with the state's inputs, and h takes its place in the state.
+int fllm_norm_short_conv(const float *x, const float *norm_w, float eps, const float *w, void *state, const int32_t *row_seg,
+                         const int32_t *slots, void *out, int rows, int width, int taps, int dtype, hipStream_t stream);
+// fllm_linear_attention: per head S <- decay_h S + k_t v_t^T, o_t = S^T q_t, token after token; S float32
+// state[slots][heads][dim][vdim].  q, k (heads * dim) and v (heads * vdim) are columns of rows of `ld` elements of `dtype`;
+// activation 1 applies silu to all three on the way in (0: none).  decay_h = decay_hi[h] + decay_lo[h] (a float pair, so that
+// the power over many tokens is that of the number itself and not of its rounding).  out float32 [rows, heads * vdim].
+int fllm_linear_attention(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
+                          float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
+                          float *out, int rows, int heads, int dim, int vdim, int activation, int dtype, hipStream_t stream);
+// out = x * rsqrt(mean x^2 + eps) * w * sigmoid(gate) over rows of `width` (w null: out = x * sigmoid(gate)); x float32 or of
+// `dtype`, gate rows of gate_ld elements and out of `dtype`.
+int fllm_gated_norm(const void *x, int x_dtype, const float *w, float eps, const void *gate, int gate_ld, void *out, int rows,
+                    int width, int dtype, hipStream_t stream);
+// out = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, powers lane by lane, N the division of a row by its root mean square (eps inside
+// the root); coeffs float32 [4] on the device.
+int fllm_polynorm(const void *z, int ld, const float *coeffs, float eps, void *out, int rows, int width, int dtype, hipStream_t stream);
+// Rows [q | k | v | ..] of `ld` elements: every head of q and k is divided by its root mean square over `norm_dim` lanes (heads
+// widened with zero lanes keep the mean of their own lanes), in place for q; k and v go into the pages of the row's request
+// (store_kv 0: q alone is normed, nothing is stored).
+int fllm_head_norm_kv_store(void *qkv, int ld, float eps, int norm_dim, const int32_t *row_pos, const int32_t *row_seg,
+                            const int32_t *tables, int table_stride, void *k_pages, void *v_pages, int rows, int heads, int kv_heads,
+                            int head_dim, int v_dim, int page_size, int key_chunk, int dtype, int store_kv, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -2,7 +2,8 @@
 // softmax over runs of 256 keys.  Used by the true 32-bit path and by the bfloat16 path for
 // shapes the MFMA kernels refuse.  Keys of `head_dim` and values of `v_dim` lanes; a row sees `window` keys back and,
 // with `chunk`, none before the start of its own chunk of positions.  A row's result depends only on its own
-// position and pages, never on the rest of the batch.
+// position and pages, never on the rest of the batch.  With `sinks` (float32, one number a head) the softmax's denominator
+// also holds exp(sinks[head]): a term without a key or a value, neither scaled nor masked, counted once.
 #include "api.h"
 #include "common.h"
 
@@ -10,7 +11,7 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
                              int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                              int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
                              int num_pages, float scale, int window, int chunk, int max_context, int single_from, void *workspace,
-                             size_t workspace_bytes, hipStream_t stream);   // attention_mfma.hip; 1: shape declined
+                             size_t workspace_bytes, const float *sinks, hipStream_t stream);   // attention_mfma.hip; 1: shape declined
 size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 
 namespace {
@@ -25,7 +26,7 @@ attention_generic_kernel(const T *__restrict__ q, int q_stride, const T *__restr
                          const T *__restrict__ v_pages, const int32_t *__restrict__ tables, int table_stride,
                          const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seg, T *__restrict__ out,
                          int heads, int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window, int chunk,
-                         int key_chunk, const float *__restrict__ head_slopes) {
+                         int key_chunk, const float *__restrict__ head_slopes, const float *__restrict__ sinks) {
     extern __shared__ float smem[];
     float *qs = smem;                   // head_dim
     float *sc = smem + head_dim;        // kBlock
@@ -85,7 +86,14 @@ attention_generic_kernel(const T *__restrict__ q, int q_stride, const T *__restr
         m = m_new;
         __syncthreads();   // sc[] is rewritten by the next chunk
     }
-    const float inv = 1.0f / l;
+    float keep = 1.0f;
+    if (sinks != nullptr) {   // a sink: one more term exp(sink) in the denominator, with no key and no value
+        const float sink = sinks[h];
+        const float m_all = fmaxf(m, sink);
+        keep = expf(m - m_all);
+        l = l * keep + expf(sink - m_all);
+    }
+    const float inv = keep / l;
 #pragma unroll
     for (int t = 0; t < kMaxDimPerThread; t++) {
         const int c = threadIdx.x + t * kBlock;
@@ -105,7 +113,7 @@ int attention_any(const void *q, int q_stride, const void *k_pages, const void *
                   const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
                   int head_dim, int v_dim, int page_size, int num_pages, float scale, int window, int chunk, int key_chunk, int dtype,
                   int max_context, int single_from, void *workspace, size_t workspace_bytes, const float *head_slopes,
-                  hipStream_t stream) {
+                  const float *sinks, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && table_stride > 0 && num_pages > 0,
                  "attention: bad sizes");
     FLLM_REQUIRE(v_dim > 0 && window >= 0 && chunk >= 0, "attention: bad value width, window or chunk");
@@ -119,7 +127,7 @@ int attention_any(const void *q, int q_stride, const void *k_pages, const void *
         const int fast = fllm_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg,
                                                   seg_start, num_segs, out, rows, heads, kv_heads, head_dim, v_dim, page_size,
                                                   num_pages, scale, window, chunk, max_context, single_from, workspace,
-                                                  workspace_bytes, stream);
+                                                  workspace_bytes, sinks, stream);
         if (fast <= 0) return fast;
     }
     FLLM_REQUIRE(v_dim <= kBlock * kMaxDimPerThread, "attention: values of %d lanes a head are more than %d", v_dim,
@@ -130,11 +138,11 @@ int attention_any(const void *q, int q_stride, const void *k_pages, const void *
     if (dtype == FLLM_F32)
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, dim3(kBlock), smem, stream, (const float *)q, q_stride,
                            (const float *)k_pages, (const float *)v_pages, tables, table_stride, row_pos, row_seg,
-                           (float *)out, heads, kv_heads, head_dim, v_dim, page_size, scale, window, chunk, key_chunk, head_slopes);
+                           (float *)out, heads, kv_heads, head_dim, v_dim, page_size, scale, window, chunk, key_chunk, head_slopes, sinks);
     else if (dtype == FLLM_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, dim3(kBlock), smem, stream, (const bf16_t *)q, q_stride,
                            (const bf16_t *)k_pages, (const bf16_t *)v_pages, tables, table_stride, row_pos, row_seg,
-                           (bf16_t *)out, heads, kv_heads, head_dim, v_dim, page_size, scale, window, chunk, key_chunk, head_slopes);
+                           (bf16_t *)out, heads, kv_heads, head_dim, v_dim, page_size, scale, window, chunk, key_chunk, head_slopes, sinks);
     else
         FLLM_REQUIRE(false, "attention: unknown dtype %d", dtype);
     return fllm_check_launch("attention");
@@ -145,11 +153,11 @@ extern "C" int fllm_attention(const void *q, int q_stride, const void *k_pages, 
                               const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
                               const int32_t *seg_start, int num_segs, void *out, int rows, int heads, int kv_heads,
                               int head_dim, int v_dim, int page_size, int num_pages, float scale, int window, int chunk,
-                              int key_chunk, int dtype, int max_context, int single_from, void *workspace, size_t workspace_bytes,
-                              hipStream_t stream) {
+                              int key_chunk, const float *sinks, int dtype, int max_context, int single_from, void *workspace,
+                              size_t workspace_bytes, hipStream_t stream) {
     return attention_any(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, seg_start, num_segs, out, rows,
                          heads, kv_heads, head_dim, v_dim, page_size, num_pages, scale, window, chunk, key_chunk, dtype, max_context,
-                         single_from, workspace, workspace_bytes, nullptr, stream);
+                         single_from, workspace, workspace_bytes, nullptr, sinks, stream);
 }
 
 extern "C" int fllm_attention_sloped(const void *q, int q_stride, const void *k_pages, const void *v_pages,
@@ -160,5 +168,5 @@ extern "C" int fllm_attention_sloped(const void *q, int q_stride, const void *k_
     FLLM_REQUIRE(head_slopes != nullptr, "attention_sloped: a slope per head is required");
     return attention_any(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, seg_start, num_segs, out, rows,
                          heads, kv_heads, head_dim, head_dim, page_size, num_pages, scale, window, 0, 8, dtype, max_context, num_segs,
-                         nullptr, 0, head_slopes, stream);
+                         nullptr, 0, head_slopes, nullptr, stream);
 }

@@ -58,7 +58,14 @@ struct AttnArgs {
     // ([row tile][key/value head][part][kPartFloats]) and are counted in `counters` ([row tile][key/value head]).
     int part_tiles;
     float *parts_ws;
+    const float *sinks;   // float32 [heads] or null: the softmax's denominator also holds exp(sinks[head])
 };
+
+// The denominator of a finished row with the sink's term: `l` is the sum of exp2(score - m_log2) over the row's keys, with
+// the scores in units of log2 (already times scale * log2 e).  A row without keys (m = -inf) gets an infinite denominator.
+__device__ __forceinline__ float with_sink(float l, float m_log2, const float *sinks, int head) {
+    return sinks == nullptr ? l : l + __builtin_amdgcn_exp2f(sinks[head] * 1.4426950408889634f - m_log2);
+}
 
 __device__ __forceinline__ bf16x8_t zero8() {
     bf16x8_t z;
@@ -255,6 +262,7 @@ attn_tile_kernel(AttnArgs p) {
         }
     }
     if (rvalid) {
+        l_run = with_sink(l_run, m_run, p.sinks, head);
         const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
         bf16_t *dst = p.out + ((size_t)(row0 + tq) * p.heads + head) * D + g * 4;
 #pragma unroll
@@ -585,6 +593,7 @@ attn_tile32_kernel(AttnArgs p) {
         }
     }
     if (rvalid) {
+        l_run = with_sink(l_run, m_run * sc, p.sinks, head);      // the maximum is in raw units here
         const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
         bf16_t *dst = p.out + ((size_t)(row0 + tq) * p.heads + head) * D + 4 * h;
 #pragma unroll
@@ -747,6 +756,7 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
         }
         const size_t hrow = (size_t)row * p.heads + kvh * G + h;
         if (live_splits == 1) {
+            l = with_sink(l, m, p.sinks, kvh * G + h);
             p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
         } else if (p.counters) {   // read by another workgroup of this launch: straight to the device's point of coherence
             __hip_atomic_store(p.ws_o + (hrow * p.splits + split) * D + d, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -820,6 +830,7 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
             load_group(s0, ms, ls, os);
             add_group(m, ms, ls, os);
         }
+        l = with_sink(l, m, p.sinks, kvh * G + qtile * 16 + qi);      // once, where the parts meet
         p.out[hrow * D + d] = (bf16_t)(l > 0.f ? acc / l : 0.f);
     }
 }
@@ -827,7 +838,7 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
 template <int D>
 __global__ void __launch_bounds__(kWave)
 attn_merge_kernel(const float *__restrict__ ws_ml, const float *__restrict__ ws_o, bf16_t *__restrict__ out, int heads,
-                  int splits) {
+                  int splits, const float *__restrict__ sinks) {
     const size_t hrow = (size_t)blockIdx.x * heads + blockIdx.y;
     float m = -INFINITY;
     for (int s = 0; s < splits; s++) m = fmaxf(m, ws_ml[(hrow * splits + s) * 2]);
@@ -836,6 +847,7 @@ attn_merge_kernel(const float *__restrict__ ws_ml, const float *__restrict__ ws_
         const float ms = ws_ml[(hrow * splits + s) * 2];
         l += ws_ml[(hrow * splits + s) * 2 + 1] * (ms == -INFINITY ? 0.f : fast_exp2(ms - m));
     }
+    l = with_sink(l, m, sinks, blockIdx.y);
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     for (int d = threadIdx.x; d < D; d += kWave) {
         float acc = 0.f;
@@ -934,7 +946,7 @@ int launch(const AttnArgs &a, int uniform_rows, int max_context, void *workspace
                            smem, stream, p, qtiles);
         if (p.splits > 1 && !p.counters)
             hipLaunchKernelGGL(attn_merge_kernel<D>, dim3(a.rows, a.heads), dim3(kWave), 0, stream, p.ws_ml, p.ws_o, a.out,
-                               a.heads, p.splits);
+                               a.heads, p.splits, p.sinks);
         return fllm_check_launch("attention_decode");
     }
     if (D >= 64 && G <= 64 && fllm_option_tile32()) {   // 128 or 256 rows per workgroup on 32x32x16 products
@@ -971,7 +983,7 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
                              int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                              int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
                              int num_pages, float scale, int window, int chunk, int max_context, int single_from, void *workspace,
-                             size_t workspace_bytes, hipStream_t stream) {
+                             size_t workspace_bytes, const float *sinks, hipStream_t stream) {
     if (!fllm_fast_kernels_enabled()) return 1;
     if (v_dim != head_dim) return 1;     // these kernels read keys and values of one width
     (void)num_pages;
@@ -1007,6 +1019,7 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
     a.counters = nullptr;
     a.part_tiles = 0;
     a.parts_ws = nullptr;
+    a.sinks = sinks;
     auto run = [&](const AttnArgs &part, int uniform) {
         if (head_dim == 32) return launch<32>(part, uniform, max_context, workspace, workspace_bytes, stream);
         if (head_dim == 64) return launch<64>(part, uniform, max_context, workspace, workspace_bytes, stream);

@@ -55,15 +55,17 @@ template <> __device__ __forceinline__ float row_dot<bf16_t>(const float *xs, co
     return wave_sum(vec ? lane_dot8(xs, w, K, lane) : lane_dot<bf16_t>(xs, w, K, lane));
 }
 
-// Router: z = W h in float32, score = sigmoid(z); the `top` largest scores of a row, ties to the lower index;
-// weights[r, k] = the score of pick k.  One workgroup a row; scores through LDS.
+// Router: z = W h in float32, score = sigmoid(z) (score_mode 0) or the softmax of z over all experts (score_mode 1); the
+// `top` largest scores of a row, ties to the lower index; weights[r, k] = the score of pick k, with `renormalize` divided by
+// the sum of the picks' scores (+ 1e-20), times route_scale.  One workgroup a row; scores through LDS.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, int E, int top, int32_t *__restrict__ ids,
-             float *__restrict__ weights) {
+             float *__restrict__ weights, int score_mode, int renormalize, float route_scale) {
     extern __shared__ float smem[];
     float *xs = smem;          // K
     float *score = smem + K;   // E
+    float *picks = score + E;  // top: the picks' scores, until their sum is known
     const size_t r = blockIdx.x;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(h[r * ldh + c]);
@@ -71,10 +73,22 @@ route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, i
     const bool vec = sizeof(T) == 2 && K % 8 == 0 && ((uintptr_t)w & 15) == 0;
     for (int e = wave; e < E; e += kWaves) {
         const float z = row_dot<T>(xs, w + (size_t)e * K, K, lane, vec);
-        if (lane == 0) score[e] = 1.0f / (1.0f + expf(-z));
+        if (lane == 0) score[e] = score_mode == 0 ? 1.0f / (1.0f + expf(-z)) : z;
     }
     __syncthreads();
     if (wave != 0) return;
+    if (score_mode == 1) {   // softmax over all experts: the largest logit, the sum in index order a lane, then across lanes
+        float top_z = -INFINITY;
+        for (int e = lane; e < E; e += kWave) top_z = fmaxf(top_z, score[e]);
+        top_z = wave_max(top_z);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += kWave) sum += expf(score[e] - top_z);
+        sum = wave_sum(sum);
+        for (int e = lane; e < E; e += kWave) score[e] = expf(score[e] - top_z) / sum;
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    float picked = 0.f;
     // one wave picks: every round the largest score not yet taken, the lowest index among equals
     for (int k = 0; k < top; k++) {
         float best = -INFINITY;
@@ -90,14 +104,18 @@ route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, i
             if (other > best || (other == best && other_at < at)) best = other, at = other_at;
         }
         if (at < 0 || at >= E) at = k;           // scores that compare with nothing (NaN rows): still an expert of the stack
+        picked += best;
         if (lane == 0) {
             ids[r * top + k] = at;
-            weights[r * top + k] = best;
-            score[at] = -INFINITY;               // scores are sigmoids: nothing real is that small
+            picks[k] = best;
+            score[at] = -INFINITY;               // scores lie in [0, 1]: nothing real is that small
         }
         __builtin_amdgcn_wave_barrier();
         __threadfence_block();
     }
+    const float factor = renormalize ? route_scale / (picked + 1e-20f) : route_scale;
+    for (int k = lane; k < top; k += kWave)
+        weights[r * top + k] = (renormalize || route_scale != 1.0f) ? picks[k] * factor : picks[k];
 }
 
 // One (row, pick) pair a workgroup row (blockIdx.y), kCols output columns a workgroup (blockIdx.x), two a wave.
@@ -183,19 +201,20 @@ expert_rows_kernel(const T *__restrict__ x, int ldx, const int32_t *__restrict__
 }  // namespace
 
 extern "C" int fllm_route_topk(const void *h, int ldh, const void *w_router, int rows, int K, int E, int top, int32_t *ids,
-                               float *weights, int dtype, hipStream_t stream) {
+                               float *weights, int score_mode, int renormalize, float route_scale, int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(score_mode == 0 || score_mode == 1, "route_topk: unknown score %d", score_mode);
     FLLM_REQUIRE(rows >= 0 && K > 0 && E > 0 && top > 0 && top <= E && ldh >= K, "route_topk: bad sizes (rows %d, width %d, %d experts, %d picked)",
                  rows, K, E, top);
     FLLM_REQUIRE(h && w_router && ids && weights, "route_topk: operands missing");
-    const size_t smem = (size_t)(K + E) * sizeof(float);
+    const size_t smem = (size_t)(K + E + top) * sizeof(float);
     FLLM_REQUIRE(smem <= 64 * 1024, "route_topk: a width of %d with %d experts does not fit into LDS", K, E);
     if (rows == 0) return 0;
     if (dtype == FLLM_F32)
         hipLaunchKernelGGL(route_kernel<float>, dim3(rows), dim3(kBlock), smem, stream, (const float *)h, ldh, (const float *)w_router, K, E,
-                           top, ids, weights);
+                           top, ids, weights, score_mode, renormalize, route_scale);
     else if (dtype == FLLM_BF16)
         hipLaunchKernelGGL(route_kernel<bf16_t>, dim3(rows), dim3(kBlock), smem, stream, (const bf16_t *)h, ldh, (const bf16_t *)w_router, K,
-                           E, top, ids, weights);
+                           E, top, ids, weights, score_mode, renormalize, route_scale);
     else
         FLLM_REQUIRE(false, "route_topk: unknown dtype %d", dtype);
     return fllm_check_launch("route_topk");

@@ -101,13 +101,19 @@ stream_add_kernel(float *__restrict__ x, const int32_t *__restrict__ ids, const 
 // next.  One workgroup a row, sums in a fixed order: a row gives the same bits whatever else is in the batch.
 template <typename B, typename T>
 __global__ void __launch_bounds__(kBlock)
-postnorm_add_kernel(float *__restrict__ x, const B *__restrict__ branch, int parts, const float *__restrict__ gain, float eps,
-                    int normalize, const float *__restrict__ next_w, float next_eps, T *__restrict__ next_out, int width) {
+postnorm_add_kernel(float *__restrict__ x, const B *__restrict__ branch, int parts, const float *__restrict__ part_weights,
+                    const float *__restrict__ gain, float eps, int normalize, const float *__restrict__ next_w, float next_eps, T *__restrict__ next_out, int width) {
     __shared__ float scratch[kWaves];
     const size_t r = blockIdx.x;
     const B *src = branch + r * parts * width;
     float *dst = x + r * width;
+    const float *pw = part_weights == nullptr ? nullptr : part_weights + r * parts;      // a weight a partial row
     auto value = [&](int c) {
+        if (pw != nullptr) {
+            float v = to_f32<B>(src[c]) * pw[0];
+            for (int k = 1; k < parts; k++) v = fmaf(to_f32<B>(src[(size_t)k * width + c]), pw[k], v);
+            return v;
+        }
         float v = to_f32<B>(src[c]);
         for (int k = 1; k < parts; k++) v += to_f32<B>(src[(size_t)k * width + c]);
         return v;
@@ -136,14 +142,15 @@ postnorm_add_kernel(float *__restrict__ x, const B *__restrict__ branch, int par
 
 }  // namespace
 
-extern "C" int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts, const float *gain, float eps, int normalize,
+extern "C" int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts, const float *part_weights, const float *gain,
+                                 float eps, int normalize,
                                  const float *next_w, float next_eps, void *next_out, int next_dtype, int rows, int width,
                                  hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && width > 0 && parts > 0, "postnorm_add: bad sizes");
     FLLM_REQUIRE(x && branch && gain && ((next_w == nullptr) == (next_out == nullptr)), "postnorm_add: operands missing");
     if (rows == 0) return 0;
 #define FLLM_POSTNORM(B, T) hipLaunchKernelGGL((postnorm_add_kernel<B, T>), dim3(rows), dim3(kBlock), 0, stream, x, (const B *)branch, \
-                                               parts, gain, eps, normalize, next_w, next_eps, (T *)next_out, width)
+                                               parts, part_weights, gain, eps, normalize, next_w, next_eps, (T *)next_out, width)
     if (branch_dtype == FLLM_F32 && next_dtype == FLLM_F32) FLLM_POSTNORM(float, float);
     else if (branch_dtype == FLLM_F32 && next_dtype == FLLM_BF16) FLLM_POSTNORM(float, bf16_t);
     else if (branch_dtype == FLLM_BF16 && next_dtype == FLLM_F32) FLLM_POSTNORM(bf16_t, float);

@@ -52,13 +52,14 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to a multiple of 64)")
     ap.add_argument("--page-size", type=int, default=16)
+    ap.add_argument("--max-requests", type=int, default=4, help="state slots: the most requests that are live at any time")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
     if 64 % args.page_size != 0:
         ap.error("--page-size must divide 64")
     print("[trace_run] loading kernels and model ...", file=sys.stderr, flush=True)
     runner = ModelRunner.from_folder(args.model, dtype=args.dtype, device=args.device, page_size=args.page_size,
-                                     max_tokens=args.max_tokens, max_requests=8)
+                                     max_tokens=args.max_tokens, max_requests=args.max_requests)
     print("[trace_run] ready", file=sys.stderr, flush=True)
     replay(runner, sys.stdin, args.out)
     return 0

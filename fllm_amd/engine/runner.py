@@ -292,6 +292,14 @@ class ModelRunner:
         if graph is None:
             graph = _DecodeGraph(self, bucket, bound, widths)
             self._graphs[key] = graph
+        if graph.graph is None and self.model.has_state:
+            # A capture runs the step once eagerly before it records it.  Pages take the same keys twice without harm; a state
+            # that a mixer carries from token to token would move twice.  Such a model captures on padding rows, which
+            # touch neither, and the step itself is the first replay.
+            graph.host_np[:] = graph.template
+            graph.device_buf.copy_(graph.host_buf, non_blocking=True)
+            graph.done.record()
+            graph.capture()
         graph.done.synchronize()                  # the previous copy out of the pinned buffer has finished
         h = graph.host_np
         h[:] = graph.template

@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 
 def load_library(build_if_missing: bool = True):
@@ -82,10 +82,18 @@ def load_library(build_if_missing: bool = True):
         "fllm_rope_kv_store": [c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_size,
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void, c_int, c_int, c_int, c_void, c_size,
                            c_void],
-        "fllm_postnorm_add": [c_void, c_void, c_int, c_int, c_void, c_float, c_int, c_void, c_float, c_void, c_int, c_int, c_int, c_void],
-        "fllm_route_topk": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_int, c_void],
+        "fllm_postnorm_add": [c_void, c_void, c_int, c_int, c_void, c_void, c_float, c_int, c_void, c_float, c_void, c_int, c_int, c_int, c_void],
+        "fllm_route_topk": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_int, c_int, c_float, c_int, c_void],
+        "fllm_short_conv": [c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void],
+        "fllm_norm_short_conv": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
+        "fllm_linear_attention": [c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_int,
+                                  c_int, c_int, c_int, c_int, c_int, c_void],
+        "fllm_gated_norm": [c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_int, c_int, c_void],
+        "fllm_polynorm": [c_void, c_int, c_void, c_float, c_void, c_int, c_int, c_int, c_void],
+        "fllm_head_norm_kv_store": [c_void, c_int, c_float, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_int,
+                                    c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_experts_gate_up": [c_void, c_int, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_void, c_float, c_float,
                                  c_float, c_int, c_void],
         "fllm_experts_down": [c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_void, c_int, c_void],
@@ -679,7 +687,7 @@ class Ops:
                   head_dim: int, page_size: int, scale: float, window: Optional[int], max_context: int,
                   uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None, single_from: Optional[int] = None,
                   head_slopes: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: Optional[int] = None,
-                  key_chunk: int = 8) -> torch.Tensor:
+                  key_chunk: int = 8, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
         """`q` may be a column slice of a wider row-major matrix (the fused qkv buffer).
         `max_context` bounds pos + 1 over the rows; the segments from `single_from` on have one row each
         (`uniform_rows` = 1 is `single_from` = 0: a decode step; by default no segment is known to).
@@ -687,7 +695,8 @@ class Ops:
         position encodings that bias scores; such a call runs the plain kernel in both precisions.
         `v_dim`: lanes of a value head where they differ from the keys' (`out` is [rows, heads * v_dim]); `chunk`: a row sees
         no key before the start of its own chunk of that many positions (chunks counted from position 0); `key_chunk`: values
-        of a key that lie together in a page.  The matrix-core kernels take v_dim == head_dim and key chunks of 8."""
+        of a key that lie together in a page.  The matrix-core kernels take v_dim == head_dim and key chunks of 8.
+        `sinks` (float32 [heads]): the softmax's denominator also holds exp(sinks[head]), a term without key or value."""
         rows = q.shape[0]
         v_dim = head_dim if v_dim is None else int(v_dim)
         chunk = int(chunk) if chunk else 0
@@ -712,7 +721,10 @@ class Ops:
             ws_ptr, ws_bytes = workspace.data_ptr(), workspace.numel() * workspace.element_size()
         q_stride = q.stride(0) if rows > 1 else heads * head_dim
         num_segs = seg_start.numel() - 1
+        if sinks is not None:
+            _dense(sinks, "sinks", torch.float32, (heads,))
         if head_slopes is not None:
+            _need(sinks is None, "biased scores come without a sink")
             _need(v_dim == head_dim and not chunk and key_chunk == 8, "biased scores come with one width of keys and values and no chunks")
             _dense(head_slopes, "head_slopes", torch.float32, (heads,))
             self._check(self.lib.fllm_attention_sloped(
@@ -726,7 +738,7 @@ class Ops:
         self._check(self.lib.fllm_attention(
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
             _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, head_dim, v_dim, page_size, num_pages,
-            float(scale), int(window) if window else 0, chunk, key_chunk, _DTYPE_CODE[q.dtype], int(max_context), int(single_from),
+            float(scale), int(window) if window else 0, chunk, key_chunk, _ptr(sinks), _DTYPE_CODE[q.dtype], int(max_context), int(single_from),
             ws_ptr, ws_bytes, self._stream()))
         return out
 
@@ -786,10 +798,11 @@ class Ops:
 
     def postnorm_add(self, x: torch.Tensor, branch: torch.Tensor, gain: torch.Tensor, eps: Optional[float], parts: int = 1,
                      next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
-                     next_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     next_out: Optional[torch.Tensor] = None, part_weights: Optional[torch.Tensor] = None) -> torch.Tensor:
         """x[r] += v * rsqrt(mean(v^2) + eps) * gain with v = the sum of the row's `parts` partial branches (`branch` is
         [rows * parts, width], a row's parts one after the other); eps None: x[r] += v * gain.  With `next_weight`, the
-        RMSNorm of the new rows (`next_eps`) goes to `next_out`."""
+        RMSNorm of the new rows (`next_eps`) goes to `next_out`.  `part_weights` (float32 [rows, parts]): part k of row r is
+        multiplied by part_weights[r, k] as it is summed."""
         rows, width = x.shape
         _dense(x, "x", torch.float32)
         _dense(branch, "branch", None, (rows * parts, width))
@@ -802,14 +815,19 @@ class Ops:
             _dense(next_out, "next_out", None, (rows, width))
             _need(next_out.dtype in _DTYPE_CODE, f"next_out dtype {next_out.dtype} unsupported")
             code = _DTYPE_CODE[next_out.dtype]
-        self._check(self.lib.fllm_postnorm_add(_ptr(x), _ptr(branch), _DTYPE_CODE[branch.dtype], int(parts), _ptr(gain),
+        if part_weights is not None:
+            _dense(part_weights, "part_weights", torch.float32, (rows, parts))
+        self._check(self.lib.fllm_postnorm_add(_ptr(x), _ptr(branch), _DTYPE_CODE[branch.dtype], int(parts), _ptr(part_weights), _ptr(gain),
                                                float(eps or 0.0), 0 if eps is None else 1, _ptr(next_weight), float(next_eps),
                                                _ptr(next_out), code, rows, width, self._stream()))
         return x
 
-    def route_topk(self, h: torch.Tensor, w_router: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor):
-        """score = sigmoid(h @ w_router.T) in float32; ids[r, k] / weights[r, k]: the expert with the k-th largest score of
-        row r (the lower index among equals) and that score."""
+    def route_topk(self, h: torch.Tensor, w_router: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor,
+                   score: str = "sigmoid", renormalize: bool = False, route_scale: float = 1.0):
+        """score = sigmoid(h @ w_router.T) in float32, or with `score` "softmax" the softmax of those logits over all experts;
+        ids[r, k] / weights[r, k]: the expert with the k-th largest score of row r (the lower index among equals) and that
+        score, with `renormalize` divided by the sum of the row's picked scores (+ 1e-20), times `route_scale`."""
+        _need(score in ("sigmoid", "softmax"), f"router score {score!r} unknown")
         rows, K = h.shape
         E = w_router.shape[0]
         _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _DTYPE_CODE, "h must be a row-major GPU matrix")
@@ -817,7 +835,8 @@ class Ops:
         _dense(ids, "ids", torch.int32, (rows, top))
         _dense(weights, "weights", torch.float32, (rows, top))
         self._check(self.lib.fllm_route_topk(_ptr(h), h.stride(0) if rows > 1 else K, _ptr(w_router), rows, K, E, int(top), _ptr(ids),
-                                             _ptr(weights), _DTYPE_CODE[h.dtype], self._stream()))
+                                             _ptr(weights), 1 if score == "softmax" else 0, 1 if renormalize else 0, float(route_scale),
+                                             _DTYPE_CODE[h.dtype], self._stream()))
         return ids, weights
 
     def experts_gate_up(self, h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, act: torch.Tensor,
@@ -886,6 +905,127 @@ class Ops:
             return False
         self._check(code)
         return True
+
+    # ---- what a sequence carries outside the pages, and the small kernels around it ---------------------------------------
+    def short_conv(self, x: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], row_seg: torch.Tensor,
+                   seg_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out[t] = x[t] + sum_j w[:, j] x[t - taps + 1 + j] over the rows of each segment, the inputs before the step's first
+        row from `state` [slots, taps - 1, width] (of x's type), which then takes the sequence's last taps - 1 inputs."""
+        rows, width = x.shape
+        taps = w.shape[1]
+        _dense(x, "x")
+        _need(x.dtype in _DTYPE_CODE, f"dtype {x.dtype} unsupported")
+        _dense(w, "w", torch.float32, (width, taps))
+        _dense(out, "out", x.dtype, (rows, width))
+        _need(out.data_ptr() != x.data_ptr(), "short_conv: rows read their neighbours, out cannot be x")
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(seg_start, "seg_start", torch.int32)
+        _dense(slots, "slots", torch.int32)
+        num_segs = seg_start.numel() - 1
+        _need(num_segs >= 1 and slots.numel() >= num_segs, "short_conv: a slot a segment")
+        if taps > 1:
+            _need(state is not None, "short_conv: the taps before a step need a state")
+            _dense(state, "state", x.dtype, (state.shape[0], taps - 1, width))
+        self._check(self.lib.fllm_short_conv(_ptr(x), _ptr(w), _ptr(state), _ptr(row_seg), _ptr(seg_start), _ptr(slots), num_segs,
+                                             _ptr(out), rows, width, taps, _DTYPE_CODE[x.dtype], self._stream()))
+        return out
+
+    def norm_short_conv(self, x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, state: Optional[torch.Tensor],
+                        row_seg: torch.Tensor, slots: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """`short_conv` of the RMSNorm of the float32 rows x in one kernel, for steps of ONE row a segment (segment s is row s)."""
+        rows, width = x.shape
+        taps = w.shape[1]
+        _dense(x, "x", torch.float32)
+        _dense(norm_weight, "norm_weight", torch.float32, (width,))
+        _dense(w, "w", torch.float32, (width, taps))
+        _dense(out, "out", None, (rows, width))
+        _need(out.dtype in _DTYPE_CODE, f"dtype {out.dtype} unsupported")
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(slots, "slots", torch.int32)
+        _need(slots.numel() >= rows, "norm_short_conv: a slot a row")
+        if taps > 1:
+            _need(state is not None, "norm_short_conv: the taps before a step need a state")
+            _dense(state, "state", out.dtype, (state.shape[0], taps - 1, width))
+        self._check(self.lib.fllm_norm_short_conv(_ptr(x), _ptr(norm_weight), float(eps), _ptr(w), _ptr(state), _ptr(row_seg), _ptr(slots),
+                                                  _ptr(out), rows, width, taps, _DTYPE_CODE[out.dtype], self._stream()))
+        return out
+
+    def linear_attention(self, qkv: torch.Tensor, decay_hi: torch.Tensor, decay_lo: torch.Tensor, state: torch.Tensor,
+                         row_seg: torch.Tensor, seg_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, heads: int,
+                         dim: int, vdim: int, activation: str = "silu") -> torch.Tensor:
+        """Per head S <- decay S + k v^T, o = S^T q, token after token; rows of `qkv` hold [q | k | v | ..] (heads * dim,
+        heads * dim, heads * vdim); S float32 state[slots, heads, dim, vdim]; out float32 [rows, heads * vdim]."""
+        rows = qkv.shape[0]
+        _need(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.dtype in _DTYPE_CODE, "qkv must be a row-major GPU matrix")
+        ld = qkv.stride(0) if rows > 1 else qkv.shape[1]
+        _need(qkv.shape[1] >= heads * (2 * dim + vdim), "qkv rows are too short")
+        _need(activation in ("silu", "none"), f"activation {activation!r} unknown")
+        _dense(decay_hi, "decay_hi", torch.float32, (heads,))
+        _dense(decay_lo, "decay_lo", torch.float32, (heads,))
+        _dense(state, "state", torch.float32, (state.shape[0], heads, dim, vdim))
+        _dense(out, "out", torch.float32, (rows, heads * vdim))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(seg_start, "seg_start", torch.int32)
+        _dense(slots, "slots", torch.int32)
+        num_segs = seg_start.numel() - 1
+        _need(num_segs >= 1 and slots.numel() >= num_segs, "linear_attention: a slot a segment")
+        elem = qkv.element_size()
+        base = qkv.data_ptr()
+        self._check(self.lib.fllm_linear_attention(base, base + heads * dim * elem, base + 2 * heads * dim * elem, ld, _ptr(decay_hi),
+                                                   _ptr(decay_lo), _ptr(state), _ptr(row_seg), _ptr(seg_start), _ptr(slots), num_segs,
+                                                   _ptr(out), rows, heads, dim, vdim, 1 if activation == "silu" else 0,
+                                                   _DTYPE_CODE[qkv.dtype], self._stream()))
+        return out
+
+    def gated_norm(self, x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out = x * rsqrt(mean x^2 + eps) * weight * sigmoid(gate) (weight None: out = x * sigmoid(gate)); `gate` may be a
+        column slice of a wider matrix."""
+        rows, width = x.shape
+        _dense(x, "x")
+        _need(x.dtype in _DTYPE_CODE, f"dtype {x.dtype} unsupported")
+        _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and tuple(gate.shape) == (rows, width) and gate.dtype == out.dtype,
+              "gate must be [rows, width] of out's type with unit column stride")
+        _dense(out, "out", None, (rows, width))
+        _need(out.dtype in _DTYPE_CODE and (x.dtype == torch.float32 or x.dtype == out.dtype), "gated_norm: x is float32 or of out's type")
+        if weight is not None:
+            _dense(weight, "weight", torch.float32, (width,))
+        self._check(self.lib.fllm_gated_norm(_ptr(x), _DTYPE_CODE[x.dtype], _ptr(weight), float(eps), _ptr(gate),
+                                             gate.stride(0) if rows > 1 else width, _ptr(out), rows, width, _DTYPE_CODE[out.dtype],
+                                             self._stream()))
+        return out
+
+    def polynorm(self, z: torch.Tensor, coeffs: torch.Tensor, eps: float, out: torch.Tensor) -> torch.Tensor:
+        """out = c0 N(z) + c1 N(z^2) + c2 N(z^3) + c3, N the division of a row by its root mean square; coeffs float32 [4]."""
+        rows, width = z.shape
+        _need(z.is_cuda and z.stride(1) == 1 and z.dtype in _DTYPE_CODE, "z must be a row-major GPU matrix")
+        _dense(coeffs, "coeffs", torch.float32, (4,))
+        _dense(out, "out", z.dtype, (rows, width))
+        self._check(self.lib.fllm_polynorm(_ptr(z), z.stride(0) if rows > 1 else width, _ptr(coeffs), float(eps), _ptr(out), rows, width,
+                                           _DTYPE_CODE[z.dtype], self._stream()))
+        return out
+
+    def head_norm_kv_store(self, qkv: torch.Tensor, eps: float, norm_dim: int, row_pos: torch.Tensor, row_seg: torch.Tensor,
+                           tables: torch.Tensor, k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], heads: int,
+                           kv_heads: int, head_dim: int, page_size: int, v_dim: Optional[int] = None, key_chunk: int = 8) -> None:
+        """Every head of q and k in the rows [q | k | v | ..] is divided by its root mean square over `norm_dim` lanes (q in
+        place); k and v go into the pages of the row's request (pages None: q alone is normed)."""
+        rows = qkv.shape[0]
+        v_dim = head_dim if v_dim is None else int(v_dim)
+        _dense(qkv, "qkv")
+        _need(qkv.dtype in _DTYPE_CODE and qkv.shape[1] >= (heads + kv_heads) * head_dim + kv_heads * v_dim, "qkv rows are too short")
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        store = k_pages is not None
+        if store:
+            num_pages = k_pages.shape[0]
+            _dense(k_pages, "k_pages", qkv.dtype, (num_pages, kv_heads, head_dim // key_chunk, page_size, key_chunk))
+            _dense(v_pages, "v_pages", qkv.dtype, (num_pages, kv_heads, v_dim, page_size))
+        self._check(self.lib.fllm_head_norm_kv_store(_ptr(qkv), qkv.shape[1], float(eps), int(norm_dim), _ptr(row_pos), _ptr(row_seg),
+                                                     _ptr(tables), tables.shape[1], _ptr(k_pages), _ptr(v_pages), rows, heads, kv_heads,
+                                                     head_dim, v_dim, page_size, key_chunk, _DTYPE_CODE[qkv.dtype], 1 if store else 0,
+                                                     self._stream()))
 
     def _talking_pages(self, k_pages, v_pages, dtype, kv_heads, k_dim, v_dim, page_size, key_chunk):
         _need(key_chunk > 0 and k_dim % key_chunk == 0, f"keys of {k_dim} values cannot lie in chunks of {key_chunk}")

@@ -1,4 +1,4 @@
-from . import attention, block, embedding, experts, mlp, norm, rope, stream, talking_attention  # noqa: F401  (register the parts)
+from . import attention, block, conv_input, embedding, experts, lightning, mlp, norm, rope, stream, talking_attention  # noqa: F401  (register the parts)
 from .base import Block, FeedForward, KVNeed, Mixer, Norm, Part, StateNeed
 from .runtime import Runtime
 

@@ -5,7 +5,11 @@ in the pages of the row's request; every row attends to the keys of its request 
 [pos - window + 1, pos] (all from 0 without a window) and, with `chunk`, to none before the start of its
 own chunk of that many positions (chunks counted from the request's first position), heads grouped over
 the key/value heads (h -> h / (heads / kv_heads)); values may have a width of their own (`value_head_dim`);
-output projection added to the residual stream, or stored as a branch for a block that norms it first
+output projection added to the residual stream, or stored as a branch for a block that norms it first.
+Options a design may ask for: `qk_norm_eps` (every head of q and of k is divided by its root mean square over the head's
+lanes, no weight; such a layer has no rotary), `sink` (a learned number a head whose exponential joins the softmax's
+denominator: a term without key or value, neither scaled nor masked), `output_gate` (the heads' outputs are multiplied lane
+by lane with sigmoid(W_g h) before the output projection; W_g rides in the q/k/v product)
 (rust/engine/src/rust_decoder.rs:8827-8835 projections, :8895-8898 rotary, :8955-8963 cache write,
 :6065-6166 scores, mask, softmax and output, :9025 and :9059 projection and residual).
 """
@@ -33,6 +37,7 @@ class PagedAttention(Mixer):
             "o": ((h, nh * dv), INIT_MATRIX),
             "q_bias": ((nh * d,), INIT_BIAS), "k_bias": ((nkv * d,), INIT_BIAS), "v_bias": ((nkv * dv,), INIT_BIAS),
             "o_bias": ((h,), INIT_BIAS),
+            "g": ((nh * dv, h), INIT_MATRIX), "sink": ((nh,), INIT_BIAS),
         }
 
     def __init__(self, spec, weights, rt):
@@ -73,6 +78,17 @@ class PagedAttention(Mixer):
             self.shape_args["v_dim"] = self.v_dim
         if self.key_chunk != self.KEY_CHUNK:
             self.shape_args["key_chunk"] = self.key_chunk
+        self.qk_norm_eps = spec.get("qk_norm_eps")
+        if self.qk_norm_eps is not None:
+            self.qk_norm_eps = float(self.qk_norm_eps)
+            if not self.qk_norm_eps > 0.0:
+                raise ValueError("the norm over a head's lanes needs a positive eps")
+            if spec.get("position") is not None:
+                raise ValueError("heads normed over their lanes come without rotary here: no kernel does both")
+        self.gated = bool(spec.get("output_gate", False))
+        if self.gated and self.qk_norm_eps is None:
+            raise ValueError("an output gate rides in the product of a layer with normed heads: ask for qk_norm_eps too")
+        self.sink = rt.vector(weights["sink"]) if spec.get("sink", False) else None
         position = spec.get("position")
         self.position = None
         if position is not None:
@@ -102,9 +118,12 @@ class PagedAttention(Mixer):
             return wide.view(heads * want, *t.shape[1:])
 
         # one matrix for q, k and v: the normed input is read once
-        self.w_qkv = torch.cat([widen(reorder(rt.matrix(weights["q"]), order_q), self.heads, d0, self.head_dim),
-                                widen(reorder(rt.matrix(weights["k"]), order_k), self.kv_heads, d0, self.head_dim),
-                                widen(rt.matrix(weights["v"]), self.kv_heads, dv0, self.v_dim)], dim=0).contiguous()
+        pieces = [widen(reorder(rt.matrix(weights["q"]), order_q), self.heads, d0, self.head_dim),
+                  widen(reorder(rt.matrix(weights["k"]), order_k), self.kv_heads, d0, self.head_dim),
+                  widen(rt.matrix(weights["v"]), self.kv_heads, dv0, self.v_dim)]
+        if self.gated:         # the gate's rows behind q, k and v: a zero lane of a widened head is gated by 1/2 and stays zero
+            pieces.append(widen(rt.matrix(weights["g"]), self.heads, dv0, self.v_dim))
+        self.w_qkv = torch.cat(pieces, dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
         if dv0 != self.v_dim:
             self.w_o = widen(self.w_o.t().contiguous(), self.heads, dv0, self.v_dim).t().contiguous()
@@ -139,9 +158,16 @@ class PagedAttention(Mixer):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
-        qkv = rt.empty((rows, (nh + nkv) * d + nkv * self.v_dim))
+        qkv = rt.empty((rows, self.w_qkv.shape[0]))
         ops.linear(h, self.w_qkv, qkv, bias=self.b_qkv)
         tables = ctx.tables[binding.group]
+        if self.qk_norm_eps is not None:
+            ops.head_norm_kv_store(qkv, self.qk_norm_eps, self.checkpoint_dims[0], ctx.row_pos, ctx.row_seg, tables,
+                                   binding.k_pages if binding.writes else None, binding.v_pages if binding.writes else None,
+                                   nh, nkv, d, binding.page_size, v_dim=self.v_dim, key_chunk=self.key_chunk)
+            gate = qkv[:, (nh + nkv) * d + nkv * self.v_dim:] if self.gated else None
+            self._attend_and_project(ctx, qkv[:, : nh * d], residual, binding, branch=branch, gate=gate)
+            return
         if self.position is not None:
             cos, sin, dims, pairing = self.position.cos, self.position.sin, self.position.dims, self.pairing
         else:
@@ -160,8 +186,8 @@ class PagedAttention(Mixer):
         form = fused_form(ops, rows, self.hidden, self.w_qkv) if hasattr(ops, "norm_qkv_rope_store") else None
         if rt.dtype != torch.bfloat16 or self.pairing != 1 or prologue is None or form is None or self.head_dim % 4 != 0:
             return False
-        if self.shape_args:
-            return False         # the fused store takes keys and values of one width, keys in chunks of 8
+        if self.shape_args or self.qk_norm_eps is not None or self.sink is not None:
+            return False         # the fused store takes keys and values of one width, keys in chunks of 8, and rotates
         norm_scale, norm_eps = prologue
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
         if self.position is not None:
@@ -194,13 +220,15 @@ class PagedAttention(Mixer):
 
     SPLIT_SINGLE_ROWS_FROM = 3072      # context length (measured: equal cost at about 4,000 keys)
 
-    def _attend_and_project(self, ctx, q, residual, binding, branch=None):
+    def _attend_and_project(self, ctx, q, residual, binding, branch=None, gate=None):
         rt, ops = self.rt, self.rt.ops
         rows = q.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
         tables = ctx.tables[binding.group]
         out = rt.empty((rows, nh * self.v_dim))
         shape_args = dict(self.shape_args, chunk=self.chunk) if self.chunk else self.shape_args
+        if self.sink is not None:
+            shape_args = dict(shape_args, sinks=self.sink)
         # Single rows behind portions of prompts: with long contexts they go to the kernel that splits a context over
         # workgroups (a second launch); with short ones they ride along in the portions' launch, which is faster then.
         single_from = ctx.single_rows_from()
@@ -216,6 +244,9 @@ class PagedAttention(Mixer):
                           out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
                           single_from=single_from,
                           workspace=ctx.attention_workspace(rt, rows, nh, nkv, d), **shape_args)
+        if gate is not None:
+            gated = rt.empty((rows, nh * self.v_dim))
+            out = ops.gated_norm(out, None, 0.0, gate, gated)
         if branch is not None:
             ops.linear(out, self.w_o, branch, bias=self.b_o)
         elif not add_and_prepare(ctx, ops, out, self.w_o, residual, self.b_o):

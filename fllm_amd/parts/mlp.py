@@ -6,7 +6,7 @@ from __future__ import annotations
 import torch
 
 from ..registry import register_part
-from .base import INIT_BIAS, INIT_MATRIX, FeedForward, add_and_prepare, fused_form, take_prepared
+from .base import INIT_BIAS, INIT_MATRIX, INIT_NORM, FeedForward, add_and_prepare, fused_form, take_prepared
 
 
 class GatedMLP(FeedForward):
@@ -172,5 +172,60 @@ class ClampedGLU(FeedForward):
         self.finish(ctx, act, residual, branch)
 
 
+class PolyNormMLP(FeedForward):
+    """x += W_down act(W_up n) with act(z) = a N(z) + b N(z^2) + c N(z^3) + e: powers lane by lane, N the division of a token's
+    vector of intermediate values by its root mean square (eps inside the root), and (a, b, c, e) the four learned numbers of
+    the tensor `act`.  The sums of squares and the division are float32."""
+    graph_safe = True
+    stores_branch = True
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        h, i = spec["hidden_size"], spec["intermediate_size"]
+        return {"up": ((i, h), INIT_MATRIX), "down": ((h, i), INIT_MATRIX), "act": ((4,), INIT_NORM)}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.eps = float(spec["eps"])
+        self.w_up = rt.matrix(weights["up"])
+        self.w_down = rt.matrix(weights["down"])
+        self.coeffs = rt.vector(weights["act"])
+        rt.tile_for_decode(self.w_down)
+        rt.tile_for_decode(self.w_up, priority=1)
+
+    def forward(self, ctx, h, residual, branch=None):
+        rt, ops = self.rt, self.rt.ops
+        rows = h.shape[0]
+        z = rt.empty((rows, self.inter))
+        ops.linear(h, self.w_up, z)
+        act = rt.empty((rows, self.inter))
+        ops.polynorm(z, self.coeffs, self.eps, act)
+        if branch is not None:
+            ops.linear(act, self.w_down, branch)
+        elif not add_and_prepare(ctx, ops, act, self.w_down, residual, None):
+            ops.linear(act, self.w_down, residual, accumulate=True)
+
+    def forward_from_residual(self, ctx, residual, norm) -> bool:
+        """Decode-sized steps in bfloat16: the norm before this part rides in the up product.  False: not taken."""
+        rt, ops = self.rt, self.rt.ops
+        rows = residual.shape[0]
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if rt.dtype != torch.bfloat16 or prologue is None or not hasattr(ops, "norm_linear"):
+            return False
+        if fused_form(ops, rows, self.hidden, self.w_up) != "resident":
+            return False
+        take_prepared(ctx, norm, residual)
+        z = rt.empty((rows, self.inter))
+        ops.norm_linear(residual, prologue[0], prologue[1], self.w_up, z)
+        act = rt.empty((rows, self.inter))
+        ops.polynorm(z, self.coeffs, self.eps, act)
+        if not add_and_prepare(ctx, ops, act, self.w_down, residual, None):
+            ops.linear(act, self.w_down, residual, accumulate=True)
+        return True
+
+
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "polynorm_mlp", PolyNormMLP)
 register_part("feed_forward", "clamped_glu", ClampedGLU)

@@ -35,4 +35,27 @@ class RMSNorm(Norm):
         return self.rt.ops.add_rmsnorm(x, branch, self.weight, self.eps, out)
 
 
+class ScalarRMSNorm(RMSNorm):
+    """RMSNorm whose weight is ONE number for all coordinates: y = x * rsqrt(mean(x^2) + eps) * g.  The number is spread over a
+    vector at load, so every kernel that takes a norm's weight vector (and every kernel that folds a norm in) serves it."""
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        return {"weight": ((), INIT_NORM)}
+
+    def __init__(self, spec, weights, rt):
+        Norm.__init__(self, spec, weights, rt)
+        self.size = int(spec["size"])
+        self.eps = float(spec["eps"])
+        if not self.eps > 0.0:
+            raise ValueError("RMSNorm needs a positive eps")
+        g = weights["weight"]
+        if g.numel() != 1:
+            raise ValueError(f"a norm with one weight for all coordinates got {g.numel()} numbers")
+        # the checkpoint's tensor is placed (the runtime knows placed tensors by their host address, so only tensors that
+        # outlive the call go through it) and spread on the device
+        self.weight = rt.vector(g).reshape(1).expand(self.size).contiguous()
+
+
 register_part("norm", "rms", RMSNorm)
+register_part("norm", "rms_scalar", ScalarRMSNorm)

@@ -207,5 +207,5 @@ def write_safetensors(path: str, tensors: Dict[str, torch.Tensor]) -> None:
         fh.write(raw)
         for t in blobs:
             if t.numel():
-                fh.write(t.view(torch.uint8).reshape(-1).numpy().tobytes() if t.dtype != torch.bool
+                fh.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.dtype != torch.bool
                          else t.to(torch.uint8).numpy().tobytes())

@@ -131,7 +131,7 @@ class ReferenceOps:
 
     def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, seg_start, out, heads, kv_heads, head_dim, page_size, scale,
                   window, max_context, uniform_rows=0, workspace=None, single_from=None, head_slopes=None, v_dim=None, chunk=None,
-                  key_chunk=8):
+                  key_chunk=8, sinks=None):
         rows = q.shape[0]
         group = heads // kv_heads
         v_dim = head_dim if v_dim is None else v_dim
@@ -155,14 +155,20 @@ class ReferenceOps:
                 s = (k[:, h // group, :] @ qr[h]) * scale
                 if head_slopes is not None:
                     s = s + float(head_slopes[h]) * (keys - pos).double()
-                p = torch.softmax(s, dim=0)
+                if sinks is not None:         # one more term in the denominator, without a value
+                    p = torch.softmax(torch.cat([s, sinks[h].double().reshape(1)]), dim=0)[:-1]
+                else:
+                    p = torch.softmax(s, dim=0)
                 out[r, h * v_dim:(h + 1) * v_dim] = (p @ v[:, h // group, :]).to(out.dtype)
         return out
 
     # ---- a branch normed on its way into the stream; routed experts ----
-    def postnorm_add(self, x, branch, gain, eps, parts=1, next_weight=None, next_eps=0.0, next_out=None):
+    def postnorm_add(self, x, branch, gain, eps, parts=1, next_weight=None, next_eps=0.0, next_out=None, part_weights=None):
         rows, width = x.shape
-        v = branch.double().view(rows, parts, width).sum(1)
+        v = branch.double().view(rows, parts, width)
+        if part_weights is not None:
+            v = v * part_weights.double().view(rows, parts, 1)
+        v = v.sum(1)
         if eps is not None:
             v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
         x.copy_((x.double() + v * gain.double()).to(x.dtype))
@@ -170,12 +176,92 @@ class ReferenceOps:
             self.rmsnorm(x, next_weight, next_eps, next_out)
         return x
 
-    def route_topk(self, h, w_router, top, ids, weights):
-        score = torch.sigmoid((h.double() @ w_router.double().T).float())
+    def route_topk(self, h, w_router, top, ids, weights, score="sigmoid", renormalize=False, route_scale=1.0):
+        z = (h.double() @ w_router.double().T).float()
+        score = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, dim=1)
         order = torch.sort(score, dim=1, descending=True, stable=True)[1][:, :top]
         ids.copy_(order.to(ids.dtype))
-        weights.copy_(torch.gather(score, 1, order))
+        picked = torch.gather(score, 1, order)
+        if renormalize:
+            picked = picked / (picked.sum(1, keepdim=True) + 1e-20)
+        weights.copy_(picked * route_scale)
         return ids, weights
+
+    # ---- what a sequence carries outside the pages: a short convolution's inputs, a linear attention's matrix ----
+    def short_conv(self, x, w, state, row_seg, seg_start, slots, out):
+        rows, width = x.shape
+        taps = w.shape[1]
+        keep = taps - 1
+        res = torch.zeros_like(out)
+        starts = [int(v) for v in seg_start]
+        for s in range(len(starts) - 1):
+            r0, r1 = starts[s], starts[s + 1]
+            if r1 <= r0 or int(row_seg[r0]) < 0:
+                continue
+            slot = int(slots[s])
+            old = state[slot].double() if keep else x.new_zeros((0, width)).double()
+            seq = torch.cat([old, x[r0:r1].double()])                      # inputs at t - keep .. t + n - 1
+            for t in range(r1 - r0):
+                acc = (seq[t:t + taps] * w.double().T).sum(0)              # w[:, j] meets the input taps - 1 - j back
+                res[r0 + t] = (x[r0 + t].double() + acc).to(out.dtype)
+            if keep:
+                state[slot] = seq[-keep:].to(state.dtype)
+        out.copy_(res)
+        return out
+
+    def linear_attention(self, qkv, decay_hi, decay_lo, state, row_seg, seg_start, slots, out, heads, dim, vdim, activation="silu"):
+        act = (lambda z: z / (1.0 + torch.exp(-z))) if activation == "silu" else (lambda z: z)
+        decay = decay_hi.double() + decay_lo.double()
+        starts = [int(v) for v in seg_start]
+        out.zero_()
+        for s in range(len(starts) - 1):
+            r0, r1 = starts[s], starts[s + 1]
+            if r1 <= r0 or int(row_seg[r0]) < 0:
+                continue
+            S = state[int(slots[s])].double()
+            for r in range(r0, r1):
+                row = qkv[r].double()
+                q = act(row[:heads * dim]).view(heads, dim)
+                k = act(row[heads * dim:2 * heads * dim]).view(heads, dim)
+                v = act(row[2 * heads * dim:2 * heads * dim + heads * vdim]).view(heads, vdim)
+                S = decay.view(heads, 1, 1) * S + k.unsqueeze(2) * v.unsqueeze(1)
+                out[r] = torch.einsum("hdv,hd->hv", S, q).reshape(-1).to(out.dtype)
+            state[int(slots[s])] = S.to(state.dtype)
+        return out
+
+    def gated_norm(self, x, weight, eps, gate, out):
+        v = x.double()
+        if weight is not None:
+            v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight.double()
+        out.copy_((v * torch.sigmoid(gate.double())).to(out.dtype))
+        return out
+
+    def polynorm(self, z, coeffs, eps, out):
+        z = z.double()
+        c = coeffs.double()
+        n = lambda t: t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps)
+        out.copy_((c[0] * n(z) + c[1] * n(z * z) + c[2] * n(z * z * z) + c[3]).to(out.dtype))
+        return out
+
+    def head_norm_kv_store(self, qkv, eps, norm_dim, row_pos, row_seg, tables, k_pages, v_pages, heads, kv_heads, head_dim,
+                           page_size, v_dim=None, key_chunk=8):
+        rows = qkv.shape[0]
+        v_dim = head_dim if v_dim is None else v_dim
+        normed = (heads + kv_heads) * head_dim
+        view = qkv[:, :normed].view(rows, heads + kv_heads, head_dim)
+        for r in range(rows):
+            seg = int(row_seg[r])
+            if seg < 0:
+                continue
+            a = view[r].double()
+            y = (a / torch.sqrt((a * a).sum(-1, keepdim=True) / norm_dim + eps)).to(qkv.dtype)
+            view[r, :heads] = y[:heads]
+            if k_pages is None:
+                continue
+            pos = int(row_pos[r])
+            page, off = int(tables[seg, pos // page_size]), pos % page_size
+            k_pages[page, :, :, off, :] = y[heads:].reshape(kv_heads, head_dim // key_chunk, key_chunk)
+            v_pages[page, :, :, off] = qkv[r, normed:normed + kv_heads * v_dim].view(kv_heads, v_dim)
 
     def experts_gate_up(self, h, ids, weights, w_gate_up, act, limit=0.0, alpha=1.0, up_offset=0.0):
         rows, top = ids.shape
