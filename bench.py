@@ -247,6 +247,23 @@ def purivik_config(size, layers):
     return cfg, layers
 
 
+def venadra_config(size, layers):
+    """`layers` layers: three with linear attention (as many heads of the same size, a state of dim x dim floats a head) and
+    then one with softmax attention over the row's chunk, a convolution of four taps before every mixer, dense (PolyNorm, two
+    matrices of the dense width) and routed feed-forwards in turn (two of eight clamped gated experts of half that width)."""
+    heads, dim = size["heads"], size["dim"]
+    linear = {"heads": heads, "dim": dim, "vdim": dim, "decay": [1.0 - 2.0 ** -(3 + 5 * h / max(1, heads - 1)) for h in range(heads)]}
+    softmax = {"heads": heads, "kv_heads": size["kv_heads"], "dim": dim, "vdim": dim, "scale": dim ** -0.5, "mask": {"size": DESIGN_CHUNK}}
+    dense = {"kind": "dense", "ff": size["ff"]}
+    routed = {"kind": "moe", "expert": {"ff": size["ff"] // DESIGN_TOP, "limit": 7.0},
+              "router": {"experts": DESIGN_EXPERTS, "top": DESIGN_TOP, "scale": 1.0}}
+    cfg = {"architecture": "Venadra", "width": size["width"], "vocab": size["vocab"], "embedding": {"scale": 1.0},
+           "norm": {"eps": 1e-5}, "canon": {"taps": 4}, "max_position": 32768,
+           "layers": [{"type": "attention" if i % 4 == 3 else "lightning", "mixer": softmax if i % 4 == 3 else linear,
+                       "mlp": routed if i % 2 else dense} for i in range(layers)]}
+    return cfg, layers
+
+
 def llama_config_of(size, layer_runs):
     return {"model_type": "llama", "architectures": ["LlamaForCausalLM"], "num_hidden_layers": layer_runs,
             "hidden_size": size["width"], "num_attention_heads": size["heads"], "num_key_value_heads": size["kv_heads"],
@@ -255,7 +272,7 @@ def llama_config_of(size, layer_runs):
 
 
 def design_run(args):
-    """Prefill and decode throughput of another design (Menitar, Purivik) beside Llama at equal sizes (width, heads, head
+    """Prefill and decode throughput of another design (Menitar, Purivik, Venadra) beside Llama at equal sizes (width, heads, head
     size, feed-forward, vocabulary, as many layers as the other has layer runs), random bfloat16 weights, with the device
     time of the kernels of a decode step and of a prefill step of each.  Prints one JSON line of its own."""
     import gc
@@ -264,7 +281,7 @@ def design_run(args):
     from fllm_amd import Engine, SamplingParams
     size = DESIGN_SIZES[args.design_size]
     layers = args.layers or size["layers"]
-    design, layer_runs = {"menitar": menitar_config, "purivik": purivik_config}[args.design](size, layers)
+    design, layer_runs = {"menitar": menitar_config, "purivik": purivik_config, "venadra": venadra_config}[args.design](size, layers)
     models = {args.design: (design, size["vocab"]), "llama": (llama_config_of(size, layer_runs), size["vocab"])}
     batches = sorted({1, args.batch, 64})
     steps, warmup = min(args.steps, 96), args.warmup
@@ -365,7 +382,7 @@ def main():
     ap.add_argument("--sampled", action="store_true",
                     help="for profiling the sampling kernels: the decode runs draw with temperature 0.8, top-k 50 and top-p 0.9 under a "
                          "repetition penalty of 1.1 and report 5 log-probabilities a token (the headline run is greedy)")
-    ap.add_argument("--design", choices=["menitar", "purivik"], default=None,
+    ap.add_argument("--design", choices=["menitar", "purivik", "venadra"], default=None,
                     help="instead of the headline run: prefill and decode of this design beside Llama at equal sizes, with the kernels' "
                          "device times of both; prints a line of its own")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="1.5b", help="with --design: the layer sizes")

@@ -346,9 +346,13 @@ int fllm_norm_short_conv(const float *x, const float *norm_w, float eps, const f
 // state[slots][heads][dim][vdim].  q, k (heads * dim) and v (heads * vdim) are columns of rows of `ld` elements of `dtype`;
 // activation 1 applies silu to all three on the way in (0: none).  decay_h = decay_hi[h] + decay_lo[h] (a float pair, so that
 // the power over many tokens is that of the number itself and not of its rounding).  out float32 [rows, heads * vdim].
+// form 0: steps with more rows than segments (portions of prompts) run chunks of 32 tokens on the matrix cores in float32 where
+// the sizes allow (dim a multiple of 16 up to 128, vdim a multiple of 16), all others token after token; 1: token after token;
+// 2: chunks, an error where the sizes do not allow them.
 int fllm_linear_attention(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
                           float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
-                          float *out, int rows, int heads, int dim, int vdim, int activation, int dtype, hipStream_t stream);
+                          float *out, int rows, int heads, int dim, int vdim, int activation, int form, int dtype,
+                          hipStream_t stream);
 // out = x * rsqrt(mean x^2 + eps) * w * sigmoid(gate) over rows of `width` (w null: out = x * sigmoid(gate)); x float32 or of
 // `dtype`, gate rows of gate_ld elements and out of `dtype`.
 int fllm_gated_norm(const void *x, int x_dtype, const float *w, float eps, const void *gate, int gate_ld, void *out, int rows,

@@ -1,0 +1,242 @@
+// Linear attention with a decay a head over portions of prompts, on the matrix cores in float32.
+//
+// The recurrence S_t = a S_(t-1) + k_t v_t^T, o_t = S_t^T q_t is taken kC = 32 tokens at a time.  With S the state before a
+// chunk of n tokens (t, s count inside the chunk):
+//     o_t = a^(t+1) S^T q_t + sum_{s <= t} a^(t-s) (q_t . k_s) v_s          S' = a^n S + sum_s a^(n-1-s) k_s v_s^T
+// which are four matrix products: the scores Q K^T (masked and decayed into P), S^T Q^T, V^T P^T, and K~^T V.  Every product
+// runs as v_mfma_f32_16x16x4_f32: the operands are float32 (the activations of q, k, v are not rounded, the scores, the
+// weights and the state stay float32), so the kernel serves both element types of the projections.
+//
+// v_mfma_f32_16x16x4_f32: lane l gives A[m = l%16][k = l/16] and B[k = l/16][n = l%16] and receives
+// D[m = 4*(l/16) + r][n = l%16] in register r.  A contraction may number its k's as it likes as long as A and B agree, so a
+// result tile is at once the A operand of a later product over its rows: register r of lane l, D[4g + r][n] with g = l/16,
+// is A[m = n][slot g] of step r, and B then brings row 4g + r of the other matrix into slot g.  The state lives in such
+// tiles for the whole call: it is the accumulator of K~^T V and the A operand of S^T Q^T, and never passes through LDS.
+//
+// One workgroup of four waves a (segment, head, 32 value lanes).  Wave w holds the state's rows of the key blocks
+// w, w + 4, .. (16 keys a block) for both 16-lane halves of the slice.  A chunk:
+//   1. q, k (32 x dim) and v (32 x 32) pass the activation into LDS; rows beyond the chunk's tokens are zeros.
+//   2. waves 0..2 take the three 16 x 16 blocks of the scores on and under the diagonal, multiply by a^(t-s), zero what
+//      lies above the diagonal and leave P in LDS; every wave multiplies its rows of the state with Q^T and leaves its
+//      part of the 32 x 32 result in LDS (in register order, so that the sum needs no index).
+//   3. wave w takes output block (w / 2, w % 2): the sum of the four parts times a^(t+1), then V^T P^T on top; the block
+//      goes to `out`.  Then every wave multiplies its state by a^n and adds K~^T V.
+// The powers a^0 .. a^32 come from the decay's float pair in double precision, once a workgroup.
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+constexpr int kC = 32;            // tokens a chunk
+constexpr int kVB = 32;           // value lanes a workgroup
+constexpr int kLDV = 48;          // row stride of V in LDS: lane groups 16 banks apart
+constexpr int kLDP = 33;
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float act_f(float z, int activation) { return activation == 1 ? z / (1.0f + expf(-z)) : z; }
+
+__host__ __device__ constexpr size_t chunked_lds_floats(int dim) {
+    return 2 * (size_t)kC * (dim + 4) + (size_t)kC * kLDV + (size_t)kC * kLDP + 4 * 4 * 4 * 64 + 40;
+}
+
+template <typename T, int NB>     // NB: key blocks a wave (dim <= 64 * NB)
+__global__ void __launch_bounds__(kThreads)
+linear_attention_chunked_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, int ld,
+                                const float *__restrict__ decay_hi, const float *__restrict__ decay_lo, float *__restrict__ state,
+                                const int32_t *__restrict__ row_seg, const int32_t *__restrict__ seg_start,
+                                const int32_t *__restrict__ slots, float *__restrict__ out, int heads, int dim, int vdim,
+                                int activation) {
+    extern __shared__ float smem[];
+    const int LDQ = dim + 4;
+    float *Qs = smem;                          // [kC][LDQ]
+    float *Ks = Qs + kC * LDQ;                 // [kC][LDQ]
+    float *Vs = Ks + kC * LDQ;                 // [kC][kLDV]
+    float *Ps = Vs + kC * kLDV;                // [kC][kLDP]
+    float *Part = Ps + kC * kLDP;              // [wave][block][register][lane]
+    float *pw = Part + 4 * 4 * 4 * 64;         // a^0 .. a^kC
+
+    const int seg = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * kVB;
+    const int r0 = seg_start[seg], n = seg_start[seg + 1] - r0;
+    if (n <= 0) return;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int ln = lane & 15, g = lane >> 4;
+    const int out_ld = heads * vdim;
+    if (row_seg[r0] < 0) {   // padding rows: no state is touched
+        for (int i = tid; i < n * kVB; i += kThreads) {
+            const int t = i / kVB, c = j0 + i % kVB;
+            if (c < vdim) out[(size_t)(r0 + t) * out_ld + (size_t)h * vdim + c] = 0.f;
+        }
+        return;
+    }
+    if (tid <= kC) pw[tid] = (float)pow((double)decay_hi[h] + (double)decay_lo[h], (double)tid);
+    const int key_blocks = dim / 16;
+    float *mine = state + ((size_t)slots[seg] * heads + h) * dim * vdim;
+
+    f32x4_t S[NB][2];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int vj = 0; vj < 2; vj++) {
+            const int di = wave + 4 * b, col = j0 + 16 * vj + ln;
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                S[b][vj][r] = (di < key_blocks && col < vdim) ? mine[(size_t)(16 * di + 4 * g + r) * vdim + col] : 0.f;
+        }
+
+    for (int c0 = 0; c0 < n; c0 += kC) {
+        const int nc = min(kC, n - c0);
+        // 1. the chunk's q, k, v into LDS
+        for (int i = tid; i < kC * dim; i += kThreads) {
+            const int t = i / dim, c = i - t * dim;
+            float qv = 0.f, kv = 0.f;
+            if (t < nc) {
+                const size_t at = (size_t)(r0 + c0 + t) * ld + (size_t)h * dim + c;
+                qv = act_f(to_f32<T>(q[at]), activation);
+                kv = act_f(to_f32<T>(k[at]), activation);
+            }
+            Qs[t * LDQ + c] = qv;
+            Ks[t * LDQ + c] = kv;
+        }
+        for (int i = tid; i < kC * kVB; i += kThreads) {
+            const int t = i / kVB, c = i % kVB;
+            float vv = 0.f;
+            if (t < nc && j0 + c < vdim) vv = act_f(to_f32<T>(v[(size_t)(r0 + c0 + t) * ld + (size_t)h * vdim + j0 + c]), activation);
+            Vs[t * kLDV + c] = vv;
+        }
+        __syncthreads();
+
+        // 2a. scores on and under the diagonal: block (ti, si) = (0, 0), (1, 0), (1, 1)
+        if (wave < 3) {
+            const int ti = wave == 0 ? 0 : 1, si = wave == 2 ? 1 : 0;
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+            const float *qrow = Qs + (16 * ti + ln) * LDQ + 4 * g, *krow = Ks + (16 * si + ln) * LDQ + 4 * g;
+            for (int j = 0; j < key_blocks; j++) {
+                const f32x4_t qa = *(const f32x4_t *)(qrow + 16 * j), kb = *(const f32x4_t *)(krow + 16 * j);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[r], kb[r], acc, 0, 0, 0);
+            }
+            const int s = 16 * si + ln;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int t = 16 * ti + 4 * g + r;
+                Ps[t * kLDP + s] = s <= t ? acc[r] * pw[t - s] : 0.f;
+            }
+        } else {   // the block above the diagonal is never read: (0, 1) stays out of every sum below
+        }
+        // 2b. this wave's rows of the state times Q^T: four blocks (value half vj, token half nj)
+        {
+            f32x4_t part[2][2];
+#pragma unroll
+            for (int vj = 0; vj < 2; vj++)
+#pragma unroll
+                for (int nj = 0; nj < 2; nj++) part[vj][nj] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const int di = wave + 4 * b;
+                if (di < key_blocks) {
+#pragma unroll
+                    for (int nj = 0; nj < 2; nj++) {
+                        const f32x4_t qb = *(const f32x4_t *)(Qs + (16 * nj + ln) * LDQ + 16 * di + 4 * g);
+#pragma unroll
+                        for (int vj = 0; vj < 2; vj++)
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                part[vj][nj] = __builtin_amdgcn_mfma_f32_16x16x4f32(S[b][vj][r], qb[r], part[vj][nj], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int vj = 0; vj < 2; vj++)
+#pragma unroll
+                for (int nj = 0; nj < 2; nj++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) Part[((wave * 4 + vj * 2 + nj) * 4 + r) * 64 + lane] = part[vj][nj][r];
+        }
+        __syncthreads();
+
+        // 3a. output block (vj, nj) of this wave: lane (ln, g), register r is o[token 16 nj + ln][value 16 vj + 4 g + r]
+        {
+            const int vj = wave >> 1, nj = wave & 1;
+            const int t = 16 * nj + ln;
+            f32x4_t o;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                float sum = 0.f;
+#pragma unroll
+                for (int w = 0; w < 4; w++) sum += Part[((w * 4 + vj * 2 + nj) * 4 + r) * 64 + lane];
+                o[r] = sum * pw[t + 1];
+            }
+            const int steps = nj == 0 ? 4 : 8;       // keys of the first half alone reach tokens of the first half
+            for (int s4 = 0; s4 < steps; s4++) {
+                const int s = 4 * s4 + g;
+                o = __builtin_amdgcn_mfma_f32_16x16x4f32(Vs[s * kLDV + 16 * vj + ln], Ps[t * kLDP + s], o, 0, 0, 0);
+            }
+            const int col = j0 + 16 * vj + 4 * g;
+            if (t < nc && col < vdim) *(f32x4_t *)(out + (size_t)(r0 + c0 + t) * out_ld + (size_t)h * vdim + col) = o;
+        }
+        // 3b. the state behind the chunk
+        {
+            const float all = pw[nc];
+            float wk[8];
+#pragma unroll
+            for (int s4 = 0; s4 < 8; s4++) {
+                const int s = 4 * s4 + g;
+                wk[s4] = s < nc ? pw[nc - 1 - s] : 0.f;
+            }
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                const int di = wave + 4 * b;
+                if (di < key_blocks) {
+#pragma unroll
+                    for (int vj = 0; vj < 2; vj++) S[b][vj] *= all;
+#pragma unroll
+                    for (int s4 = 0; s4 < 8; s4++) {
+                        const int s = 4 * s4 + g;
+                        const float ka = Ks[s * LDQ + 16 * di + ln] * wk[s4];
+#pragma unroll
+                        for (int vj = 0; vj < 2; vj++)
+                            S[b][vj] = __builtin_amdgcn_mfma_f32_16x16x4f32(ka, Vs[s * kLDV + 16 * vj + ln], S[b][vj], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        __syncthreads();      // the next chunk overwrites what this one read
+    }
+
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int vj = 0; vj < 2; vj++) {
+            const int di = wave + 4 * b, col = j0 + 16 * vj + ln;
+            if (di < key_blocks && col < vdim)
+#pragma unroll
+                for (int r = 0; r < 4; r++) mine[(size_t)(16 * di + 4 * g + r) * vdim + col] = S[b][vj][r];
+        }
+}
+
+}  // namespace
+
+// 0: launched; 1: the sizes are not this kernel's (keys in blocks of 16 up to 128 lanes, values in blocks of 16).
+int fllm_linear_attention_chunked(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
+                                  float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
+                                  float *out, int rows, int heads, int dim, int vdim, int activation, int dtype, hipStream_t stream) {
+    if (dim % 16 != 0 || dim > 128 || vdim % 16 != 0) return 1;
+    const int slices = (vdim + kVB - 1) / kVB;
+    if (slices > 65535 || heads > 65535) return 1;
+    const size_t smem = chunked_lds_floats(dim) * sizeof(float);
+    if (smem > 64 * 1024) return 1;
+    const dim3 grid(num_segs, heads, slices);
+#define FLLM_CHUNKED(T, NB)                                                                                                       \
+    hipLaunchKernelGGL((linear_attention_chunked_kernel<T, NB>), grid, dim3(kThreads), smem, stream, (const T *)q, (const T *)k, \
+                       (const T *)v, ld, decay_hi, decay_lo, state, row_seg, seg_start, slots, out, heads, dim, vdim, activation)
+    if (dtype == FLLM_F32) {
+        if (dim <= 64) FLLM_CHUNKED(float, 1);
+        else FLLM_CHUNKED(float, 2);
+    } else if (dtype == FLLM_BF16) {
+        if (dim <= 64) FLLM_CHUNKED(bf16_t, 1);
+        else FLLM_CHUNKED(bf16_t, 2);
+    } else
+        return 1;
+#undef FLLM_CHUNKED
+    return 0;
+}

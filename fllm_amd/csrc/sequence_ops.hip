@@ -12,6 +12,11 @@
 #include "api.h"
 #include "common.h"
 
+int fllm_linear_attention_chunked(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
+                                  float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
+                                  float *out, int rows, int heads, int dim, int vdim, int activation, int dtype,
+                                  hipStream_t stream);   // linear_attention_mfma.hip; 1: sizes declined
+
 namespace {
 
 constexpr int kBlock = 256;
@@ -312,13 +317,22 @@ extern "C" int fllm_norm_short_conv(const float *x, const float *norm_w, float e
 
 extern "C" int fllm_linear_attention(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
                                      float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots,
-                                     int num_segs, float *out, int rows, int heads, int dim, int vdim, int activation, int dtype,
-                                     hipStream_t stream) {
+                                     int num_segs, float *out, int rows, int heads, int dim, int vdim, int activation, int form,
+                                     int dtype, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && dim > 0 && vdim > 0 && num_segs > 0 && ld > 0, "linear_attention: bad sizes");
     FLLM_REQUIRE(q && k && v && decay_hi && decay_lo && state && row_seg && seg_start && slots && out, "linear_attention: operands missing");
     FLLM_REQUIRE(activation == 0 || activation == 1, "linear_attention: unknown activation %d", activation);
     FLLM_REQUIRE(heads <= 65535, "linear_attention: too many heads");
+    FLLM_REQUIRE(form >= 0 && form <= 2, "linear_attention: unknown form %d", form);
+    FLLM_REQUIRE(dtype == FLLM_F32 || dtype == FLLM_BF16, "linear_attention: unknown dtype %d", dtype);
     if (rows == 0) return 0;
+    // a step that holds more rows than segments holds portions of prompts: those go over the matrix cores a chunk at a time
+    if (form == 2 || (form == 0 && rows > num_segs)) {
+        const int declined = fllm_linear_attention_chunked(q, k, v, ld, decay_hi, decay_lo, state, row_seg, seg_start, slots, num_segs,
+                                                           out, rows, heads, dim, vdim, activation, dtype, stream);
+        if (!declined) return fllm_check_launch("linear_attention_chunked");
+        FLLM_REQUIRE(form != 2, "linear_attention: heads of %d and %d lanes are not the chunked kernel's", dim, vdim);
+    }
     // the widest slice of value lanes whose share of the state fits into LDS beside q, k and the partial sums
     int VB = 64;
     while (VB / 2 >= vdim && VB > 1) VB >>= 1;

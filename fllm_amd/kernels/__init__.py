@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 
 def load_library(build_if_missing: bool = True):
@@ -89,7 +89,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_short_conv": [c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_norm_short_conv": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_linear_attention": [c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_int,
-                                  c_int, c_int, c_int, c_int, c_int, c_void],
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_gated_norm": [c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_int, c_int, c_void],
         "fllm_polynorm": [c_void, c_int, c_void, c_float, c_void, c_int, c_int, c_int, c_void],
         "fllm_head_norm_kv_store": [c_void, c_int, c_float, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_int,
@@ -952,14 +952,17 @@ class Ops:
 
     def linear_attention(self, qkv: torch.Tensor, decay_hi: torch.Tensor, decay_lo: torch.Tensor, state: torch.Tensor,
                          row_seg: torch.Tensor, seg_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, heads: int,
-                         dim: int, vdim: int, activation: str = "silu") -> torch.Tensor:
-        """Per head S <- decay S + k v^T, o = S^T q, token after token; rows of `qkv` hold [q | k | v | ..] (heads * dim,
-        heads * dim, heads * vdim); S float32 state[slots, heads, dim, vdim]; out float32 [rows, heads * vdim]."""
+                         dim: int, vdim: int, activation: str = "silu", form: str = "auto") -> torch.Tensor:
+        """Per head S <- decay S + k v^T, o = S^T q over each segment's rows; rows of `qkv` hold [q | k | v | ..] (heads * dim,
+        heads * dim, heads * vdim); S float32 state[slots, heads, dim, vdim]; out float32 [rows, heads * vdim].  `form`:
+        "tokens" runs token after token, "chunks" 32 tokens at a time on the matrix cores in float32 (dim a multiple of 16 up
+        to 128, vdim a multiple of 16), "auto" chunks where a step holds portions of prompts and the sizes allow."""
         rows = qkv.shape[0]
         _need(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.dtype in _DTYPE_CODE, "qkv must be a row-major GPU matrix")
         ld = qkv.stride(0) if rows > 1 else qkv.shape[1]
         _need(qkv.shape[1] >= heads * (2 * dim + vdim), "qkv rows are too short")
         _need(activation in ("silu", "none"), f"activation {activation!r} unknown")
+        _need(form in ("auto", "tokens", "chunks"), f"form {form!r} unknown")
         _dense(decay_hi, "decay_hi", torch.float32, (heads,))
         _dense(decay_lo, "decay_lo", torch.float32, (heads,))
         _dense(state, "state", torch.float32, (state.shape[0], heads, dim, vdim))
@@ -974,7 +977,7 @@ class Ops:
         self._check(self.lib.fllm_linear_attention(base, base + heads * dim * elem, base + 2 * heads * dim * elem, ld, _ptr(decay_hi),
                                                    _ptr(decay_lo), _ptr(state), _ptr(row_seg), _ptr(seg_start), _ptr(slots), num_segs,
                                                    _ptr(out), rows, heads, dim, vdim, 1 if activation == "silu" else 0,
-                                                   _DTYPE_CODE[qkv.dtype], self._stream()))
+                                                   {"auto": 0, "tokens": 1, "chunks": 2}[form], _DTYPE_CODE[qkv.dtype], self._stream()))
         return out
 
     def gated_norm(self, x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -108,6 +108,10 @@ def weights(cfg, seed, decided_router=False):
             out[p + "canon1"] = rng.normal(0, 0.3, (W, taps))
         out[p + "mix.q"] = rng.normal(0, 2 * W ** -0.5, (H * d, W))
         out[p + "mix.k"] = rng.normal(0, 2 * W ** -0.5, (G * d, W))
+        if spec["type"] == "lightning":
+            # keys lean towards their own queries: a token's product with itself is then well above the rounding of its
+            # terms, so the sign of a first token's output (all a norm over the heads keeps of it) is no close call
+            out[p + "mix.k"] = 0.6 * out[p + "mix.q"] + 0.8 * out[p + "mix.k"]
         out[p + "mix.v"] = rng.normal(0, W ** -0.5, (G * dv, W))
         out[p + "mix.g"] = rng.normal(0, 2 * W ** -0.5, (H * dv, W))
         out[p + "mix.o"] = quiet(rng.normal(0, (H * dv) ** -0.5, (W, H * dv)))
