@@ -15,7 +15,8 @@
 //
 // One workgroup of four waves a (segment, head, 32 value lanes).  Wave w holds the state's rows of the key blocks
 // w, w + 4, .. (16 keys a block) for both 16-lane halves of the slice.  A chunk:
-//   1. q, k (32 x dim) and v (32 x 32) pass the activation into LDS; rows beyond the chunk's tokens are zeros.
+//   1. q, k (32 x dim) and v (32 x 32), loaded 16 bytes at a time while the chunk before was computed, pass the activation
+//      into LDS; rows beyond the chunk's tokens are zeros.
 //   2. waves 0..2 take the three 16 x 16 blocks of the scores on and under the diagonal, multiply by a^(t-s), zero what
 //      lies above the diagonal and leave P in LDS; every wave multiplies its rows of the state with Q^T and leaves its
 //      part of the 32 x 32 result in LDS (in register order, so that the sum needs no index).
@@ -33,7 +34,15 @@ constexpr int kLDV = 48;          // row stride of V in LDS: lane groups 16 bank
 constexpr int kLDP = 33;
 constexpr int kThreads = 256;
 
-__device__ __forceinline__ float act_f(float z, int activation) { return activation == 1 ? z / (1.0f + expf(-z)) : z; }
+// silu of a projection: float32 rows get the library's exponential and a division; bfloat16 rows, whose own rounding is
+// 2^-9, the hardware's exponential and reciprocal (a few units in the last place of a float), a quarter of the instructions
+template <typename T> __device__ __forceinline__ float act_f(float z, int activation);
+template <> __device__ __forceinline__ float act_f<float>(float z, int activation) {
+    return activation == 1 ? z / (1.0f + expf(-z)) : z;
+}
+template <> __device__ __forceinline__ float act_f<bf16_t>(float z, int activation) {
+    return activation == 1 ? z * __frcp_rn(1.0f + __expf(-z)) : z;
+}
 
 __host__ __device__ constexpr size_t chunked_lds_floats(int dim) {
     return 2 * (size_t)kC * (dim + 4) + (size_t)kC * kLDV + (size_t)kC * kLDP + 4 * 4 * 4 * 64 + 40;
@@ -83,38 +92,83 @@ linear_attention_chunked_kernel(const T *__restrict__ q, const T *__restrict__ k
                 S[b][vj][r] = (di < key_blocks && col < vdim) ? mine[(size_t)(16 * di + 4 * g + r) * vdim + col] : 0.f;
         }
 
+    // 1. the chunk's q, k, v: 16 bytes a load, all of a thread's loads in flight at once, and the next chunk's loads issued
+    // before this chunk's products, so that a chunk waits for memory once at most
+    constexpr int EPV = 16 / (int)sizeof(T);                                  // elements a load
+    constexpr int QV = (kC * 64 * NB / EPV + kThreads - 1) / kThreads;        // loads a thread for q, and for k
+    constexpr int VV = (kC * kVB / EPV + kThreads - 1) / kThreads;
+    const int dimv = dim / EPV;
+    uint4 rq[QV], rk[QV], rv[VV];
+    int tq[QV], cq[QV];                  // a load's token and first lane: the same in every chunk
+#pragma unroll
+    for (int it = 0; it < QV; it++) {
+        const int i = tid + it * kThreads;
+        tq[it] = i / dimv;
+        cq[it] = (i - tq[it] * dimv) * EPV;
+    }
+    auto issue = [&](int c0) {
+        const int nc = min(kC, n - c0);
+#pragma unroll
+        for (int it = 0; it < QV; it++) {
+            rq[it] = rk[it] = uint4{0u, 0u, 0u, 0u};
+            if (tq[it] < nc) {
+                const size_t at = (size_t)(r0 + c0 + tq[it]) * ld + (size_t)h * dim + cq[it];
+                rq[it] = *(const uint4 *)(q + at);
+                rk[it] = *(const uint4 *)(k + at);
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < VV; it++) {
+            const int i = tid + it * kThreads, t = i / (kVB / EPV), cv = i % (kVB / EPV);
+            rv[it] = uint4{0u, 0u, 0u, 0u};
+            if (t < nc && j0 + cv * EPV < vdim)
+                rv[it] = *(const uint4 *)(v + (size_t)(r0 + c0 + t) * ld + (size_t)h * vdim + j0 + cv * EPV);
+        }
+    };
+    // through the activation into LDS, four lanes a store; rows beyond the chunk's tokens were loaded as zeros
+    auto put = [&](float *dst, const uint4 &raw) {
+        const T *e = (const T *)&raw;
+#pragma unroll
+        for (int e4 = 0; e4 < EPV; e4 += 4) {
+            f32x4_t a;
+#pragma unroll
+            for (int x = 0; x < 4; x++) a[x] = act_f<T>(to_f32<T>(e[e4 + x]), activation);
+            *(f32x4_t *)(dst + e4) = a;
+        }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int it = 0; it < QV; it++)
+            if (tq[it] < kC) {
+                put(Qs + tq[it] * LDQ + cq[it], rq[it]);
+                put(Ks + tq[it] * LDQ + cq[it], rk[it]);
+            }
+#pragma unroll
+        for (int it = 0; it < VV; it++) {
+            const int i = tid + it * kThreads, t = i / (kVB / EPV), cv = i % (kVB / EPV);
+            if (t < kC) put(Vs + t * kLDV + cv * EPV, rv[it]);
+        }
+    };
+    issue(0);
     for (int c0 = 0; c0 < n; c0 += kC) {
         const int nc = min(kC, n - c0);
-        // 1. the chunk's q, k, v into LDS
-        for (int i = tid; i < kC * dim; i += kThreads) {
-            const int t = i / dim, c = i - t * dim;
-            float qv = 0.f, kv = 0.f;
-            if (t < nc) {
-                const size_t at = (size_t)(r0 + c0 + t) * ld + (size_t)h * dim + c;
-                qv = act_f(to_f32<T>(q[at]), activation);
-                kv = act_f(to_f32<T>(k[at]), activation);
-            }
-            Qs[t * LDQ + c] = qv;
-            Ks[t * LDQ + c] = kv;
-        }
-        for (int i = tid; i < kC * kVB; i += kThreads) {
-            const int t = i / kVB, c = i % kVB;
-            float vv = 0.f;
-            if (t < nc && j0 + c < vdim) vv = act_f(to_f32<T>(v[(size_t)(r0 + c0 + t) * ld + (size_t)h * vdim + j0 + c]), activation);
-            Vs[t * kLDV + c] = vv;
-        }
+        commit();
+        if (c0 + kC < n) issue(c0 + kC);
         __syncthreads();
 
         // 2a. scores on and under the diagonal: block (ti, si) = (0, 0), (1, 0), (1, 1)
         if (wave < 3) {
             const int ti = wave == 0 ? 0 : 1, si = wave == 2 ? 1 : 0;
-            f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+            f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};      // two chains: a product does not wait for the one before
             const float *qrow = Qs + (16 * ti + ln) * LDQ + 4 * g, *krow = Ks + (16 * si + ln) * LDQ + 4 * g;
             for (int j = 0; j < key_blocks; j++) {
                 const f32x4_t qa = *(const f32x4_t *)(qrow + 16 * j), kb = *(const f32x4_t *)(krow + 16 * j);
-#pragma unroll
-                for (int r = 0; r < 4; r++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[r], kb[r], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[0], kb[0], acc, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[1], kb[1], acc1, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[2], kb[2], acc, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[3], kb[3], acc1, 0, 0, 0);
             }
+            acc += acc1;
             const int s = 16 * si + ln;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
@@ -216,11 +270,15 @@ linear_attention_chunked_kernel(const T *__restrict__ q, const T *__restrict__ k
 
 }  // namespace
 
-// 0: launched; 1: the sizes are not this kernel's (keys in blocks of 16 up to 128 lanes, values in blocks of 16).
+// 0: launched; 1: the sizes are not this kernel's (keys in blocks of 16 up to 128 lanes, values in blocks of 16, rows that
+// begin on 16 bytes).
 int fllm_linear_attention_chunked(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
                                   float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
                                   float *out, int rows, int heads, int dim, int vdim, int activation, int dtype, hipStream_t stream) {
     if (dim % 16 != 0 || dim > 128 || vdim % 16 != 0) return 1;
+    // rows are read 16 bytes at a time
+    const int epv = dtype == FLLM_F32 ? 4 : 8;
+    if (ld % epv != 0 || (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) != 0) return 1;
     const int slices = (vdim + kVB - 1) / kVB;
     if (slices > 65535 || heads > 65535) return 1;
     const size_t smem = chunked_lds_floats(dim) * sizeof(float);

@@ -5,7 +5,8 @@
 //   short_conv          y_t = x_t + sum_j w[:, j] x_(t - taps + 1 + j): a causal convolution over time on every channel, the
 //                       last taps - 1 inputs of a sequence kept in its state slot.
 //   linear_attention    S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head, S float32 [dim][vdim] in the sequence's
-//                       state slot; q, k and v pass through an activation on the way in.
+//                       state slot; q, k and v pass through an activation on the way in.  Token after token, the state in
+//                       registers (values in groups of four lanes) or in LDS (any sizes).
 //   gated_norm          out = x * rsqrt(mean x^2 + eps) * w * sigmoid(gate) (w absent: out = x * sigmoid(gate)).
 //   polynorm            out = a N(z) + b N(z^2) + c N(z^3) + e, N the division by a row's root mean square.
 //   head_norm_kv_store  q and k divided by their root mean square over a head's lanes, k and v stored into the pages.
@@ -82,9 +83,11 @@ short_conv_state_kernel(const T *__restrict__ x, T *__restrict__ state, const in
     }
 }
 
-// The norm before the convolution and the convolution in one pass, for steps of one row a segment: one workgroup a row.  The
-// normed row is rounded to T before it is used, as the norm kernel's output would be, so that a token gives the same bits
-// whether it came alone or in a portion.  A thread owns a channel of the state: it reads the old entries before it writes.
+// The norm before the convolution and the convolution in one pass, for steps of one row a segment: one workgroup a row and
+// block of kBlock channels; every workgroup of a row sums the row's squares itself (in the norm kernel's order), so that no
+// thread loops over channels and all it reads is on its way at once.  The normed value is rounded to T before it is used, as
+// the norm kernel's output would be, so that a token gives the same bits whether it came alone or in a portion.  A thread
+// owns a channel of the state: it reads the old entries before it writes any.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 norm_short_conv_kernel(const float *__restrict__ x, const float *__restrict__ norm_w, float eps, const float *__restrict__ w,
@@ -92,32 +95,38 @@ norm_short_conv_kernel(const float *__restrict__ x, const float *__restrict__ no
                        T *__restrict__ out, int width, int taps) {
     __shared__ float scratch[kWaves];
     const int r = blockIdx.x;
+    const int c = blockIdx.y * kBlock + threadIdx.x;
     const int seg = row_seg[r];
     if (seg < 0) {   // padding row
-        for (int c = threadIdx.x; c < width; c += kBlock) out[(size_t)r * width + c] = from_f32<T>(0.f);
+        if (c < width) out[(size_t)r * width + c] = from_f32<T>(0.f);
         return;
     }
     const float *src = x + (size_t)r * width;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < width; c += kBlock) ss = fmaf(src[c], src[c], ss);
+#pragma unroll 8
+    for (int i = threadIdx.x; i < width; i += kBlock) ss = fmaf(src[i], src[i], ss);
     ss = block_sum<kWaves>(ss, scratch);
+    if (c >= width) return;
     const float inv = 1.0f / sqrtf(ss / (float)width + eps);
     const int keep = taps - 1;
     T *mine = state + (size_t)slots[seg] * keep * width;
-    for (int c = threadIdx.x; c < width; c += kBlock) {
-        const float *wc = w + (size_t)c * taps;
-        const T h = from_f32<T>(src[c] * (inv * norm_w[c]));
-        const float now = to_f32<T>(h);
-        float acc = 0.f;
-        for (int i = 0; i < keep; i++) {          // oldest input first; entry i moves to i - 1
-            const T old = mine[(size_t)i * width + c];
-            acc = fmaf(wc[i], to_f32<T>(old), acc);
-            if (i > 0) mine[(size_t)(i - 1) * width + c] = old;
-        }
-        if (keep > 0) mine[(size_t)(keep - 1) * width + c] = h;
-        acc = fmaf(wc[taps - 1], now, acc);
-        out[(size_t)r * width + c] = from_f32<T>(now + acc);
+    const float *wc = w + (size_t)c * taps;
+    T held[kMaxKeep];
+#pragma unroll
+    for (int i = 0; i < kMaxKeep; i++)
+        if (i < keep) held[i] = mine[(size_t)i * width + c];
+    const T h = from_f32<T>(src[c] * (inv * norm_w[c]));
+    const float now = to_f32<T>(h);
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxKeep; i++) {      // oldest input first; entry i moves to i - 1
+        if (i >= keep) break;
+        acc = fmaf(wc[i], to_f32<T>(held[i]), acc);
+        if (i > 0) mine[(size_t)(i - 1) * width + c] = held[i];
     }
+    if (keep > 0) mine[(size_t)(keep - 1) * width + c] = h;
+    acc = fmaf(wc[taps - 1], now, acc);
+    out[(size_t)r * width + c] = from_f32<T>(now + acc);
 }
 
 // ---- linear attention, one token after the other ----------------------------------------------------------------------------
@@ -178,6 +187,92 @@ linear_attention_kernel(const T *__restrict__ q, const T *__restrict__ k, const 
         for (int i = g; i < dim; i += G) mine[(size_t)i * vdim + j0 + j] = S[i * VB + j];
 }
 
+// The same recurrence with the state in registers, for values in groups of four lanes and keys of up to 32 * RP lanes: one
+// workgroup a (segment, head, slice of 32 value lanes), thread (g, j4) owns rows g, g + 32, .. of the four columns at 4 * j4.
+// The state is read once, 16 bytes a thread and 128 bytes a row, and written once behind the segment's last token, which is
+// all a decode step does; the sum over the rows is taken over the lanes of a wave and then over the four waves, in an order
+// that no size of the batch changes.
+constexpr int kRowsVB = 32;
+template <typename T, int RP>
+__global__ void __launch_bounds__(kBlock)
+linear_attention_rows_kernel(const T *__restrict__ q, const T *__restrict__ k, const T *__restrict__ v, int ld,
+                             const float *__restrict__ decay_hi, const float *__restrict__ decay_lo, float *__restrict__ state,
+                             const int32_t *__restrict__ row_seg, const int32_t *__restrict__ seg_start,
+                             const int32_t *__restrict__ slots, float *__restrict__ out, int heads, int dim, int vdim,
+                             int activation) {
+    constexpr int G = kBlock / (kRowsVB / 4);      // 32 groups of rows
+    __shared__ float qs[G * RP], ks[G * RP];
+    __shared__ f32x4_t part[kWaves][kRowsVB / 4];
+    const int seg = blockIdx.x, h = blockIdx.y, j0 = blockIdx.z * kRowsVB;
+    const int r0 = seg_start[seg], n = seg_start[seg + 1] - r0;
+    if (n <= 0) return;
+    const int tid = threadIdx.x, j4 = tid & 7, g = tid >> 3;
+    const int col = j0 + 4 * j4;
+    const bool live = col < vdim;
+    const size_t out_ld = (size_t)heads * vdim;
+    if (row_seg[r0] < 0) {   // padding rows: no state is touched
+        if (g == 0 && live)
+            for (int t = 0; t < n; t++) *(f32x4_t *)(out + (size_t)(r0 + t) * out_ld + (size_t)h * vdim + col) = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        return;
+    }
+    float *mine = state + ((size_t)slots[seg] * heads + h) * dim * vdim;
+    f32x4_t S[RP];
+#pragma unroll
+    for (int p = 0; p < RP; p++) {
+        const int i = g + G * p;
+        S[p] = (live && i < dim) ? *(const f32x4_t *)(mine + (size_t)i * vdim + col) : f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    const float dh = decay_hi[h], dl = decay_lo[h];
+    for (int t = 0; t < n; t++) {
+        const size_t row = (size_t)(r0 + t) * ld;
+        if (t > 0) __syncthreads();      // the token before has read qs, ks and part
+        for (int c = tid; c < dim; c += kBlock) {
+            qs[c] = activate(to_f32<T>(q[row + (size_t)h * dim + c]), activation);
+            ks[c] = activate(to_f32<T>(k[row + (size_t)h * dim + c]), activation);
+        }
+        f32x4_t vv = {0.f, 0.f, 0.f, 0.f};
+        if (live)
+#pragma unroll
+            for (int e = 0; e < 4; e++) vv[e] = activate(to_f32<T>(v[row + (size_t)h * vdim + col + e]), activation);
+        __syncthreads();
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < RP; p++) {
+            const int i = g + G * p;
+            if (i < dim) {
+                const float kk = ks[i], qq = qs[i];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float s = S[p][e];
+                    s = fmaf(s, dh, fmaf(s, dl, kk * vv[e]));
+                    S[p][e] = s;
+                    acc[e] = fmaf(s, qq, acc[e]);
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) {      // the eight row groups of a wave: lanes 8, 16 and 32 apart hold the same columns
+            acc[e] += __shfl_xor(acc[e], 8, kWave);
+            acc[e] += __shfl_xor(acc[e], 16, kWave);
+            acc[e] += __shfl_xor(acc[e], 32, kWave);
+        }
+        if ((tid & (kWave - 1)) < 8) part[tid / kWave][j4] = acc;
+        __syncthreads();
+        if (tid < 8 && live) {
+            f32x4_t o = part[0][tid];
+#pragma unroll
+            for (int a = 1; a < kWaves; a++) o += part[a][tid];
+            *(f32x4_t *)(out + (size_t)(r0 + t) * out_ld + (size_t)h * vdim + col) = o;
+        }
+    }
+    if (live)
+#pragma unroll
+        for (int p = 0; p < RP; p++) {
+            const int i = g + G * p;
+            if (i < dim) *(f32x4_t *)(mine + (size_t)i * vdim + col) = S[p];
+        }
+}
+
 // ---- gated norm ---------------------------------------------------------------------------------------------------------------
 template <typename X, typename T>
 __global__ void __launch_bounds__(kBlock)
@@ -189,6 +284,7 @@ gated_norm_kernel(const X *__restrict__ x, const float *__restrict__ w, float ep
     float inv = 1.0f;
     if (w != nullptr) {
         float ss = 0.f;
+#pragma unroll 8      // eight loads on their way at once: a row is a few values a thread and waits for memory, not for arithmetic
         for (int c = threadIdx.x; c < width; c += kBlock) {
             const float a = to_f32<X>(src[c]);
             ss = fmaf(a, a, ss);
@@ -196,6 +292,7 @@ gated_norm_kernel(const X *__restrict__ x, const float *__restrict__ w, float ep
         ss = block_sum<kWaves>(ss, scratch);
         inv = 1.0f / sqrtf(ss / (float)width + eps);
     }
+#pragma unroll 8
     for (int c = threadIdx.x; c < width; c += kBlock) {
         float a = to_f32<X>(src[c]) * inv;
         if (w != nullptr) a *= w[c];
@@ -211,6 +308,7 @@ polynorm_kernel(const T *__restrict__ z, int ld, const float *__restrict__ coeff
     const size_t r = blockIdx.x;
     const T *src = z + r * ld;
     float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll 8      // eight loads on their way at once
     for (int c = threadIdx.x; c < width; c += kBlock) {
         const float a = to_f32<T>(src[c]), a2 = a * a, a3 = a2 * a;
         s2 += a2;
@@ -223,6 +321,7 @@ polynorm_kernel(const T *__restrict__ z, int ld, const float *__restrict__ coeff
     const float n = (float)width;
     const float c1 = coeffs[0] / sqrtf(s2 / n + eps), c2 = coeffs[1] / sqrtf(s4 / n + eps), c3 = coeffs[2] / sqrtf(s6 / n + eps);
     const float c0 = coeffs[3];
+#pragma unroll 8
     for (int c = threadIdx.x; c < width; c += kBlock) {
         const float a = to_f32<T>(src[c]);
         out[r * width + c] = from_f32<T>(fmaf(a, fmaf(a, fmaf(a, c3, c2), c1), c0));
@@ -301,14 +400,14 @@ extern "C" int fllm_short_conv(const void *x, const float *w, void *state, const
 
 extern "C" int fllm_norm_short_conv(const float *x, const float *norm_w, float eps, const float *w, void *state, const int32_t *row_seg,
                                     const int32_t *slots, void *out, int rows, int width, int taps, int dtype, hipStream_t stream) {
-    FLLM_REQUIRE(rows >= 0 && width > 0 && taps >= 1 && eps > 0.f, "norm_short_conv: bad sizes");
+    FLLM_REQUIRE(rows >= 0 && width > 0 && taps >= 1 && taps - 1 <= kMaxKeep && eps > 0.f, "norm_short_conv: bad sizes");
     FLLM_REQUIRE(x && norm_w && w && out && row_seg && slots && (state || taps == 1), "norm_short_conv: operands missing");
     if (rows == 0) return 0;
     if (dtype == FLLM_F32)
-        hipLaunchKernelGGL(norm_short_conv_kernel<float>, dim3(rows), dim3(kBlock), 0, stream, x, norm_w, eps, w, (float *)state, row_seg,
+        hipLaunchKernelGGL(norm_short_conv_kernel<float>, dim3(rows, (width + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, x, norm_w, eps, w, (float *)state, row_seg,
                            slots, (float *)out, width, taps);
     else if (dtype == FLLM_BF16)
-        hipLaunchKernelGGL(norm_short_conv_kernel<bf16_t>, dim3(rows), dim3(kBlock), 0, stream, x, norm_w, eps, w, (bf16_t *)state, row_seg,
+        hipLaunchKernelGGL(norm_short_conv_kernel<bf16_t>, dim3(rows, (width + kBlock - 1) / kBlock), dim3(kBlock), 0, stream, x, norm_w, eps, w, (bf16_t *)state, row_seg,
                            slots, (bf16_t *)out, width, taps);
     else
         FLLM_REQUIRE(false, "norm_short_conv: unknown dtype %d", dtype);
@@ -332,6 +431,25 @@ extern "C" int fllm_linear_attention(const void *q, const void *k, const void *v
                                                            out, rows, heads, dim, vdim, activation, dtype, stream);
         if (!declined) return fllm_check_launch("linear_attention_chunked");
         FLLM_REQUIRE(form != 2, "linear_attention: heads of %d and %d lanes are not the chunked kernel's", dim, vdim);
+    }
+    // values in groups of four lanes: the state passes through registers
+    if (vdim % 4 == 0 && dim <= 256) {
+        const dim3 grid(num_segs, heads, (vdim + kRowsVB - 1) / kRowsVB);
+#define FLLM_ROWS(T, RP)                                                                                                          \
+    hipLaunchKernelGGL((linear_attention_rows_kernel<T, RP>), grid, dim3(kBlock), 0, stream, (const T *)q, (const T *)k,          \
+                       (const T *)v, ld, decay_hi, decay_lo, state, row_seg, seg_start, slots, out, heads, dim, vdim, activation)
+#define FLLM_ROWS_OF(T)                                                                                                           \
+    do {                                                                                                                          \
+        if (dim <= 32) FLLM_ROWS(T, 1);                                                                                           \
+        else if (dim <= 64) FLLM_ROWS(T, 2);                                                                                      \
+        else if (dim <= 128) FLLM_ROWS(T, 4);                                                                                     \
+        else FLLM_ROWS(T, 8);                                                                                                     \
+    } while (0)
+        if (dtype == FLLM_F32) FLLM_ROWS_OF(float);
+        else FLLM_ROWS_OF(bf16_t);
+#undef FLLM_ROWS_OF
+#undef FLLM_ROWS
+        return fllm_check_launch("linear_attention_rows");
     }
     // the widest slice of value lanes whose share of the state fits into LDS beside q, k and the partial sums
     int VB = 64;
