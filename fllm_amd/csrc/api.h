@@ -348,11 +348,14 @@ int fllm_norm_short_conv(const float *x, const float *norm_w, float eps, const f
 // the power over many tokens is that of the number itself and not of its rounding).  out float32 [rows, heads * vdim].
 // form 0: steps with more rows than segments (portions of prompts) run chunks of 32 tokens on the matrix cores in float32 where
 // the sizes allow (dim a multiple of 16 up to 128, vdim a multiple of 16), all others token after token; 1: token after token;
-// 2: chunks, an error where the sizes do not allow them.
+// 2: chunks, an error where the sizes do not allow them.  `carried` (null, or fllm_linear_attention_carried_floats floats):
+// with it, the chunked form cuts the segments of a step of 512 rows or more into parts of 256 tokens that run side by side,
+// each from zeros, and a second kernel hands the states from part to part and adds what the tokens of a part lack.
 int fllm_linear_attention(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
                           float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
                           float *out, int rows, int heads, int dim, int vdim, int activation, int form, int dtype,
-                          hipStream_t stream);
+                          float *carried, hipStream_t stream);
+size_t fllm_linear_attention_carried_floats(int rows, int num_segs, int heads, int dim, int vdim);
 // out = x * rsqrt(mean x^2 + eps) * w * sigmoid(gate) over rows of `width` (w null: out = x * sigmoid(gate)); x float32 or of
 // `dtype`, gate rows of gate_ld elements and out of `dtype`.
 int fllm_gated_norm(const void *x, int x_dtype, const float *w, float eps, const void *gate, int gate_ld, void *out, int rows,

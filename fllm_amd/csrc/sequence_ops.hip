@@ -15,7 +15,7 @@
 
 int fllm_linear_attention_chunked(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
                                   float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots, int num_segs,
-                                  float *out, int rows, int heads, int dim, int vdim, int activation, int dtype,
+                                  float *out, int rows, int heads, int dim, int vdim, int activation, int dtype, float *carried,
                                   hipStream_t stream);   // linear_attention_mfma.hip; 1: sizes declined
 
 namespace {
@@ -417,7 +417,7 @@ extern "C" int fllm_norm_short_conv(const float *x, const float *norm_w, float e
 extern "C" int fllm_linear_attention(const void *q, const void *k, const void *v, int ld, const float *decay_hi, const float *decay_lo,
                                      float *state, const int32_t *row_seg, const int32_t *seg_start, const int32_t *slots,
                                      int num_segs, float *out, int rows, int heads, int dim, int vdim, int activation, int form,
-                                     int dtype, hipStream_t stream) {
+                                     int dtype, float *carried, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && dim > 0 && vdim > 0 && num_segs > 0 && ld > 0, "linear_attention: bad sizes");
     FLLM_REQUIRE(q && k && v && decay_hi && decay_lo && state && row_seg && seg_start && slots && out, "linear_attention: operands missing");
     FLLM_REQUIRE(activation == 0 || activation == 1, "linear_attention: unknown activation %d", activation);
@@ -428,7 +428,7 @@ extern "C" int fllm_linear_attention(const void *q, const void *k, const void *v
     // a step that holds more rows than segments holds portions of prompts: those go over the matrix cores a chunk at a time
     if (form == 2 || (form == 0 && rows > num_segs)) {
         const int declined = fllm_linear_attention_chunked(q, k, v, ld, decay_hi, decay_lo, state, row_seg, seg_start, slots, num_segs,
-                                                           out, rows, heads, dim, vdim, activation, dtype, stream);
+                                                           out, rows, heads, dim, vdim, activation, dtype, carried, stream);
         if (!declined) return fllm_check_launch("linear_attention_chunked");
         FLLM_REQUIRE(form != 2, "linear_attention: heads of %d and %d lanes are not the chunked kernel's", dim, vdim);
     }

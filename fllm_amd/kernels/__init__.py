@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 
 def load_library(build_if_missing: bool = True):
@@ -89,7 +89,7 @@ def load_library(build_if_missing: bool = True):
         "fllm_short_conv": [c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_norm_short_conv": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void],
         "fllm_linear_attention": [c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_int,
-                                  c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+                                  c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void],
         "fllm_gated_norm": [c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_int, c_int, c_int, c_void],
         "fllm_polynorm": [c_void, c_int, c_void, c_float, c_void, c_int, c_int, c_int, c_void],
         "fllm_head_norm_kv_store": [c_void, c_int, c_float, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_int,
@@ -162,6 +162,8 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_set_fast_kernels.restype = None
     lib.fllm_experts_grouped_plane_floats.argtypes = [c_int, c_int, c_int, c_int]
     lib.fllm_experts_grouped_plane_floats.restype = c_size
+    lib.fllm_linear_attention_carried_floats.argtypes = [c_int, c_int, c_int, c_int, c_int]
+    lib.fllm_linear_attention_carried_floats.restype = c_size
     lib.fllm_experts_grouped_work_ints.argtypes = [c_int, c_int]
     lib.fllm_experts_grouped_work_ints.restype = c_size
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -950,13 +952,17 @@ class Ops:
                                                   _ptr(out), rows, width, taps, _DTYPE_CODE[out.dtype], self._stream()))
         return out
 
+    LINEAR_ATTENTION_PARTS_ROWS = 512      # steps of this many rows and more cut their segments into parts
+
     def linear_attention(self, qkv: torch.Tensor, decay_hi: torch.Tensor, decay_lo: torch.Tensor, state: torch.Tensor,
                          row_seg: torch.Tensor, seg_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, heads: int,
-                         dim: int, vdim: int, activation: str = "silu", form: str = "auto") -> torch.Tensor:
+                         dim: int, vdim: int, activation: str = "silu", form: str = "auto", parts: bool = True) -> torch.Tensor:
         """Per head S <- decay S + k v^T, o = S^T q over each segment's rows; rows of `qkv` hold [q | k | v | ..] (heads * dim,
         heads * dim, heads * vdim); S float32 state[slots, heads, dim, vdim]; out float32 [rows, heads * vdim].  `form`:
         "tokens" runs token after token, "chunks" 32 tokens at a time on the matrix cores in float32 (dim a multiple of 16 up
-        to 128, vdim a multiple of 16), "auto" chunks where a step holds portions of prompts and the sizes allow."""
+        to 128, vdim a multiple of 16), "auto" chunks where a step holds portions of prompts and the sizes allow.  With `parts`
+        the chunked form cuts the segments of a step of 512 rows or more into parts of 256 tokens that run side by side, each
+        from zeros, and a second kernel hands the states from part to part and adds what the tokens of a part lack."""
         rows = qkv.shape[0]
         _need(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.dtype in _DTYPE_CODE, "qkv must be a row-major GPU matrix")
         ld = qkv.stride(0) if rows > 1 else qkv.shape[1]
@@ -974,10 +980,15 @@ class Ops:
         _need(num_segs >= 1 and slots.numel() >= num_segs, "linear_attention: a slot a segment")
         elem = qkv.element_size()
         base = qkv.data_ptr()
+        carried = None
+        if parts and form != "tokens" and rows >= self.LINEAR_ATTENTION_PARTS_ROWS and rows > num_segs:
+            need = int(self.lib.fllm_linear_attention_carried_floats(rows, num_segs, heads, dim, vdim))
+            carried = torch.empty((need,), dtype=torch.float32, device=qkv.device)
         self._check(self.lib.fllm_linear_attention(base, base + heads * dim * elem, base + 2 * heads * dim * elem, ld, _ptr(decay_hi),
                                                    _ptr(decay_lo), _ptr(state), _ptr(row_seg), _ptr(seg_start), _ptr(slots), num_segs,
                                                    _ptr(out), rows, heads, dim, vdim, 1 if activation == "silu" else 0,
-                                                   {"auto": 0, "tokens": 1, "chunks": 2}[form], _DTYPE_CODE[qkv.dtype], self._stream()))
+                                                   {"auto": 0, "tokens": 1, "chunks": 2}[form], _DTYPE_CODE[qkv.dtype], _ptr(carried),
+                                                   self._stream()))
         return out
 
     def gated_norm(self, x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, gate: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

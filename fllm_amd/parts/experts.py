@@ -48,6 +48,9 @@ class RoutedExperts(FeedForward):
         self.weight_on = spec.get("weight_on", "input")
         if self.weight_on not in ("input", "output"):
             raise ValueError(f"a pick's weight goes on the expert's input or output, not on {self.weight_on!r}")
+        # forward(..., branch=t) stores the picks' outputs in t; with the weights on the outputs the sum needs the weights,
+        # so this part then adds to the stream itself (an arrangement hands it a stand-in)
+        self.stores_branch = self.weight_on == "input"
         self.limit = float(spec.get("limit") or 0.0)          # 0: nothing is clamped
         self.alpha = float(spec.get("alpha", 1.0))
         self.up_offset = float(spec.get("up_offset", 0.0))
@@ -56,12 +59,6 @@ class RoutedExperts(FeedForward):
         self.w_gate_up = torch.stack([torch.cat([rt.matrix(weights[f"gate_{e}"]), rt.matrix(weights[f"up_{e}"])], dim=0)
                                       for e in range(n)]).contiguous()
         self.w_down = torch.stack([rt.matrix(weights[f"down_{e}"]) for e in range(n)]).contiguous()
-
-    @property
-    def stores_branch(self) -> bool:
-        """forward(..., branch=t) stores the picks' outputs in t; with the weights on the outputs the sum needs the weights,
-        so this part then adds to the stream itself (an arrangement hands it a stand-in)."""
-        return self.weight_on == "input"
 
     @property
     def branch_parts(self) -> int:

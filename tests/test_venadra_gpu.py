@@ -162,7 +162,7 @@ def test_a_key_far_back_is_felt_by_its_decay(ops, form, decay):
     hi, lo = decay_pair([decay, decay])
     direction = torch.randn(dim, generator=gen(2))
     direction = direction / direction.norm()
-    for target in (0, 31, 32, 33, 350, n - 1):
+    for target in (0, 31, 32, 33, 255, 256, 350, n - 1):        # a whole prompt of 700 tokens runs in parts of 256
         qkv = 1e-3 * torch.randn(n, heads * (2 * dim + vdim), generator=gen(3))
         qkv[target, heads * dim + dim:heads * dim + 2 * dim] = 6 * direction            # key of head 1
         qkv[n - 1, dim:2 * dim] = 6 * direction                                         # query of head 1
@@ -179,6 +179,38 @@ def test_a_key_far_back_is_felt_by_its_decay(ops, form, decay):
                                      out[a:b], heads, dim, vdim, activation="none", form=form if b - a > 1 else "tokens")
             # the other keys are small, not nothing: their sum is the floor under a key that has all but decayed away
             close(out[n - 1, vdim:], want, 2e-3, 2e-3 * decay ** (n - 1 - target) + 5e-4, f"key at {target}, cut at {cut}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 64, 64), (3, 128, 48), (2, 128, 128), (1, 32, 16)])
+def test_long_segments_run_in_parts(ops, ref, shape, dtype):
+    """A step of 512 rows and more cuts its segments into parts of 256 tokens that start from zeros; a second kernel hands the
+    states on and adds what the tokens lack.  Segments of one part, of a part and one token, of two parts exactly, of several
+    with a short last one, beside padding rows and single tokens; a second step goes on from the first's state."""
+    heads, dim, vdim = shape
+    hi, lo = decay_pair([1.0, 0.97, 0.9990234375][:heads])
+    segments = [700, 1, 300, -5, 256, 257, 512, 2, 1000]
+    row_seg, seg_start = rows_of(segments)
+    rows = int(seg_start[-1])
+    slots = torch.tensor([5, 0, 7, 8, 2, 1, 4, 3, 6], dtype=torch.int32)
+    state = 0.1 * torch.randn(10, heads, dim, vdim, generator=gen(1))
+    want_state, got_state, single_state = state.double(), state.clone().to(DEV), state.clone().to(DEV)
+    for step in range(2):
+        qkv = (0.2 * torch.randn(rows, heads * (2 * dim + vdim), generator=gen(10 + step))).to(dtype)
+        want = torch.empty(rows, heads * vdim, dtype=torch.float64)
+        ref.linear_attention(qkv.double(), hi, lo, want_state, row_seg, seg_start, slots, want, heads, dim, vdim)
+        args = (qkv.to(DEV), hi.to(DEV), lo.to(DEV))
+        where = (row_seg.to(DEV), seg_start.to(DEV), slots.to(DEV))
+        got = torch.full((rows, heads * vdim), 7.0, dtype=torch.float32, device=DEV)
+        ops.linear_attention(*args, got_state, *where, got, heads, dim, vdim, form="chunks")
+        single = torch.empty_like(got)
+        ops.linear_attention(*args, single_state, *where, single, heads, dim, vdim, form="chunks", parts=False)
+        scale = want.abs().max().item()
+        close(got, want, 3e-5, 3e-5 * scale, f"step {step}")
+        close(got, single, 1e-5, 1e-5 * scale, f"step {step}: parts against one pass")
+        close(got_state, want_state, 3e-5, 3e-5 * want_state.abs().max().item(), f"state behind step {step}")
+        assert not torch.equal(got, single), "the step was meant to run in parts"
+    assert torch.equal(got_state[[8, 9]].cpu(), state[[8, 9]]), "slots of no segment and of padding stay"
 
 
 def test_chunks_and_tokens_agree_and_a_row_does_not_depend_on_the_batch(ops):
@@ -479,6 +511,23 @@ def test_decode_graphs_and_eager_steps_agree(models, tmp_path, name, dtype):
             assert np.array_equal(a, b), f"{rid}: graph and eager steps differ in float32"
         else:
             assert np.abs(a - b).max() <= TOL[dtype] * np.abs(want).max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_whole_and_in_portions(models, tmp_path, dtype):
+    """1,100 tokens in one step (the linear attention runs in parts of 256 tokens), in two portions, and with the last 40
+    decoded one by one."""
+    folder, cfg, _, _, w64 = models["D", dtype]
+    toks = vc.random_ids(1100, cfg["vocab"], 77)
+    want = {"long": pv.forward(cfg, w64, toks)}
+    from fllm_amd.engine import StepEntry
+    for cuts in ([1100], [600, 500], [1060] + [1] * 40):
+        runner = make_runner(folder, dtype, 16, 1152, max_context=2048)
+        got, at = [], 0
+        for n in cuts:
+            got.append(runner.step([StepEntry("long", toks[at:at + n], list(range(n)))]).float().cpu().numpy())
+            at += n
+        check({"long": np.concatenate(got)}, want, dtype, f"long-prompt-{len(cuts)} D {dtype}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
