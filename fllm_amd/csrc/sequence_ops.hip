@@ -27,7 +27,8 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 __device__ __forceinline__ float activate(float z, int activation) { return activation == 1 ? z * sigmoid_f(z) : z; }
 
 // ---- short convolution ----------------------------------------------------------------------------------------------------
-// One workgroup a row.  The input `d` tokens back is a row of this step while the step holds it, else an entry of the state:
+// One workgroup a row (a step of prompts has rows enough to fill the device; the loop takes any number of blocks of channels
+// a row).  The input `d` tokens back is a row of this step while the step holds it, else an entry of the state:
 // state[slot][i] is the input at position (tokens before this step) - (taps - 1) + i, zeros before the sequence's start.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
@@ -36,12 +37,12 @@ short_conv_kernel(const T *__restrict__ x, const float *__restrict__ w, const T 
     const int r = blockIdx.x;
     const int seg = row_seg[r];
     if (seg < 0) {   // padding row
-        for (int c = threadIdx.x; c < width; c += kBlock) out[(size_t)r * width + c] = from_f32<T>(0.f);
+        for (int c = blockIdx.y * kBlock + threadIdx.x; c < width; c += gridDim.y * kBlock) out[(size_t)r * width + c] = from_f32<T>(0.f);
         return;
     }
     const int t = r - seg_start[seg];
     const T *mine = state + (size_t)slots[seg] * (taps - 1) * width;
-    for (int c = threadIdx.x; c < width; c += kBlock) {
+    for (int c = blockIdx.y * kBlock + threadIdx.x; c < width; c += gridDim.y * kBlock) {      // one channel a thread
         const float *wc = w + (size_t)c * taps;
         const float now = to_f32<T>(x[(size_t)r * width + c]);
         float acc = 0.f;
@@ -55,7 +56,7 @@ short_conv_kernel(const T *__restrict__ x, const float *__restrict__ w, const T 
     }
 }
 
-// One workgroup a segment, after the rows have been computed: the state becomes the last taps - 1 inputs of the sequence.
+// One workgroup a segment and block of channels, after the rows have been computed: the state becomes the last taps - 1 inputs of the sequence.
 // A thread owns a channel: it reads what it keeps of the old entries before it writes any.
 constexpr int kMaxKeep = 15;
 template <typename T>
@@ -67,7 +68,7 @@ short_conv_state_kernel(const T *__restrict__ x, T *__restrict__ state, const in
     if (n <= 0 || row_seg[r0] < 0) return;   // nothing of this segment in the step, or padding rows
     const int keep = taps - 1;
     T *mine = state + (size_t)slots[seg] * keep * width;
-    for (int c = threadIdx.x; c < width; c += kBlock) {
+    for (int c = blockIdx.y * kBlock + threadIdx.x; c < width; c += gridDim.y * kBlock) {      // one channel a thread
         T held[kMaxKeep];
 #pragma unroll
         for (int i = 0; i < kMaxKeep; i++) {
@@ -103,8 +104,13 @@ norm_short_conv_kernel(const float *__restrict__ x, const float *__restrict__ no
     }
     const float *src = x + (size_t)r * width;
     float ss = 0.f;
-#pragma unroll 8
-    for (int i = threadIdx.x; i < width; i += kBlock) ss = fmaf(src[i], src[i], ss);
+    for (int i0 = threadIdx.x; i0 < width; i0 += 4 * kBlock) {      // four loads on their way at once, summed in the row's order
+        float a[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) a[j] = i0 + j * kBlock < width ? src[i0 + j * kBlock] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) ss = fmaf(a[j], a[j], ss);
+    }
     ss = block_sum<kWaves>(ss, scratch);
     if (c >= width) return;
     const float inv = 1.0f / sqrtf(ss / (float)width + eps);
@@ -284,10 +290,13 @@ gated_norm_kernel(const X *__restrict__ x, const float *__restrict__ w, float ep
     float inv = 1.0f;
     if (w != nullptr) {
         float ss = 0.f;
-#pragma unroll 8      // eight loads on their way at once: a row is a few values a thread and waits for memory, not for arithmetic
-        for (int c = threadIdx.x; c < width; c += kBlock) {
-            const float a = to_f32<X>(src[c]);
-            ss = fmaf(a, a, ss);
+        // four loads on their way at once: a row is a few values a thread and waits for memory, not for arithmetic
+        for (int c0 = threadIdx.x; c0 < width; c0 += 4 * kBlock) {
+            float a[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) a[j] = c0 + j * kBlock < width ? to_f32<X>(src[c0 + j * kBlock]) : 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) ss = fmaf(a[j], a[j], ss);
         }
         ss = block_sum<kWaves>(ss, scratch);
         inv = 1.0f / sqrtf(ss / (float)width + eps);
@@ -381,17 +390,18 @@ extern "C" int fllm_short_conv(const void *x, const float *w, void *state, const
     FLLM_REQUIRE(taps >= 1 && taps - 1 <= kMaxKeep, "short_conv: %d taps are outside 1..%d", taps, kMaxKeep + 1);
     FLLM_REQUIRE(x && w && out && row_seg && seg_start && slots && (state || taps == 1), "short_conv: operands missing");
     if (rows == 0) return 0;
+    const int blocks = (width + kBlock - 1) / kBlock < 65535 ? (width + kBlock - 1) / kBlock : 65535;      // blocks of channels
     if (dtype == FLLM_F32) {
-        hipLaunchKernelGGL(short_conv_kernel<float>, dim3(rows), dim3(kBlock), 0, stream, (const float *)x, w, (const float *)state,
+        hipLaunchKernelGGL(short_conv_kernel<float>, dim3(rows, 1), dim3(kBlock), 0, stream, (const float *)x, w, (const float *)state,
                            row_seg, seg_start, slots, (float *)out, width, taps);
         if (taps > 1)
-            hipLaunchKernelGGL(short_conv_state_kernel<float>, dim3(num_segs), dim3(kBlock), 0, stream, (const float *)x,
+            hipLaunchKernelGGL(short_conv_state_kernel<float>, dim3(num_segs, blocks), dim3(kBlock), 0, stream, (const float *)x,
                                (float *)state, row_seg, seg_start, slots, width, taps);
     } else if (dtype == FLLM_BF16) {
-        hipLaunchKernelGGL(short_conv_kernel<bf16_t>, dim3(rows), dim3(kBlock), 0, stream, (const bf16_t *)x, w, (const bf16_t *)state,
+        hipLaunchKernelGGL(short_conv_kernel<bf16_t>, dim3(rows, 1), dim3(kBlock), 0, stream, (const bf16_t *)x, w, (const bf16_t *)state,
                            row_seg, seg_start, slots, (bf16_t *)out, width, taps);
         if (taps > 1)
-            hipLaunchKernelGGL(short_conv_state_kernel<bf16_t>, dim3(num_segs), dim3(kBlock), 0, stream, (const bf16_t *)x,
+            hipLaunchKernelGGL(short_conv_state_kernel<bf16_t>, dim3(num_segs, blocks), dim3(kBlock), 0, stream, (const bf16_t *)x,
                                (bf16_t *)state, row_seg, seg_start, slots, width, taps);
     } else
         FLLM_REQUIRE(false, "short_conv: unknown dtype %d", dtype);
