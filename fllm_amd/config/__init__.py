@@ -1,8 +1,9 @@
 from .spec import ConfigError, LayerSpec, ModelSpec, PartSpec, RunEntry, default_run_order
 from .files import read_config_json
+from .dumizen import DumizenConfig
 from .llama import LlamaConfig, RopeScaling
 from .menitar import MenitarConfig
 from .purivik import PurivikConfig
 
 __all__ = ["ConfigError", "LayerSpec", "ModelSpec", "PartSpec", "RunEntry", "default_run_order",
-           "LlamaConfig", "MenitarConfig", "PurivikConfig", "RopeScaling", "read_config_json"]
+           "DumizenConfig", "LlamaConfig", "MenitarConfig", "PurivikConfig", "RopeScaling", "read_config_json"]

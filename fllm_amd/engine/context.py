@@ -22,6 +22,8 @@ class CacheBinding:
     page_size: int
     writes: bool                            # False: the entry reads another entry's cache
     state: object = None                    # [max_requests, *shape], or name -> such a tensor: mixers with fixed-size state
+    pool_k: Optional[torch.Tensor] = None   # [pages, kv_heads, slots, k_dim] float32: means of blocks of keys (KVNeed.pooled)
+    pool_v: Optional[torch.Tensor] = None   # [pages, kv_heads, slots, v_dim] float32
 
 
 @dataclass

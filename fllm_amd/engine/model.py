@@ -22,6 +22,7 @@ class GroupKey(NamedTuple):
     v_dim: int
     window: Optional[int]
     key_chunk: int
+    pooled: int = 0
 
 
 class Model:
@@ -89,7 +90,7 @@ class Model:
                 self.entry_group[i] = self.entry_group[src]
                 self.entry_index[i] = self.entry_index[src]
                 continue
-            key = GroupKey(need.kv_heads, need.k_dim, need.v_dim, need.window, need.key_chunk)
+            key = GroupKey(need.kv_heads, need.k_dim, need.v_dim, need.window, need.key_chunk, need.pooled)
             if key not in keys:
                 keys.append(key)
                 members.append([])
@@ -107,7 +108,9 @@ class Model:
     def cache_bytes_per_page(self, page_size: int) -> List[int]:
         """Bytes a page of each group costs (keys and values of all the group's run entries)."""
         elem = torch.empty((), dtype=self.rt.dtype).element_size()
-        return [len(m) * k.kv_heads * (k.k_dim + k.v_dim) * page_size * elem for k, m in zip(self.group_keys, self.group_members)]
+        pooled = lambda k: 4 * -(-page_size // k.pooled) if k.pooled else 0       # float32 means of the blocks that end in a page
+        return [len(m) * k.kv_heads * (k.k_dim + k.v_dim) * (page_size * elem + pooled(k))
+                for k, m in zip(self.group_keys, self.group_members)]
 
     def allocate_caches(self, page_size: int, pages_per_group: Sequence[int], max_requests: int,
                         max_step_tokens: Optional[int] = None) -> CacheManager:
@@ -119,9 +122,13 @@ class Model:
             raise ValueError(f"{len(groups)} cache groups need {len(groups)} page counts")
         self.page_size = page_size
         self.null_pages = [int(n) for n in pages_per_group]
-        self.k_store, self.v_store = [], []
+        self.k_store, self.v_store, self.pool_store = [], [], []
         for g, n in zip(groups, pages_per_group):
             need = self.kv_needs[g.entries[0]]            # the group's entries agree on what they need
+            slots = need.pool_slots(page_size)
+            self.pool_store.append(None if not slots else tuple(
+                torch.zeros((len(g.entries), n + 1, g.kv_heads, slots, width), dtype=torch.float32, device=rt.device)
+                for width in (g.k_dim, g.v_dim)))
             self.k_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, *need.key_page_shape(page_size)),
                                             dtype=rt.dtype, device=rt.device))
             self.v_store.append(torch.zeros((len(g.entries), n + 1, g.kv_heads, g.v_dim, page_size),
@@ -138,8 +145,11 @@ class Model:
                                                   writes=False, state=state))
                 continue
             idx = self.entry_index[i]
+            pools = self.pool_store[g]
             self.bindings.append(CacheBinding(group=g, k_pages=self.k_store[g][idx], v_pages=self.v_store[g][idx],
-                                              page_size=page_size, writes=entry.reads_cache_of is None, state=state))
+                                              page_size=page_size, writes=entry.reads_cache_of is None, state=state,
+                                              pool_k=None if pools is None else pools[0][idx],
+                                              pool_v=None if pools is None else pools[1][idx]))
         return CacheManager(groups, list(pages_per_group), max_requests, max_step_tokens=max_step_tokens)
 
     def state_arenas(self):

@@ -1,1 +1,1 @@
-from . import llama, menitar, purivik, venadra  # noqa: F401  (register the architectures)
+from . import dumizen, llama, menitar, purivik, venadra  # noqa: F401  (register the architectures)

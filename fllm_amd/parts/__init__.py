@@ -1,4 +1,5 @@
-from . import attention, block, conv_input, embedding, experts, lightning, mlp, norm, rope, stream, talking_attention  # noqa: F401  (register the parts)
+from . import (attention, block, conv_input, embedding, experts, lightning, mlp, norm, normed_attention, pair, rope, sigmoid_attention,
+               stream, talking_attention)  # noqa: F401  (register the parts)
 from .base import Block, FeedForward, KVNeed, Mixer, Norm, Part, StateNeed
 from .runtime import Runtime
 

@@ -73,12 +73,16 @@ class KVNeed:
     out; 0: the mixer caches keys alone); `window` keys back (the token itself included) or all of them when None.
     The pages are shaped from both widths; what a mixer's kernels can read is the mixer's matter.  `key_chunk`: 0 stores
     a token's keys together ([page][kv_head][token][k_dim]); n > 0 stores them in chunks of n values, chunk by chunk over
-    the tokens of a page ([page][kv_head][k_dim / n][token][n]), the order this library's attention kernels read."""
+    the tokens of a page ([page][kv_head][k_dim / n][token][n]), the order this library's attention kernels read.
+    `pooled`: n > 0 keeps, beside every page, the float32 means of the keys and of the values of each block of n positions
+    that ends in the page ([page][kv_head][slot][k_dim or v_dim], slot = (the block's last position % page_size) / n): what
+    a mixer reads of blocks that a window has passed.  Such a cache keeps every page (no `window`)."""
     kv_heads: int
     k_dim: int
     v_dim: Optional[int] = None
     window: Optional[int] = None
     key_chunk: int = 0
+    pooled: int = 0
 
     def __post_init__(self):
         if self.v_dim is None:
@@ -87,6 +91,12 @@ class KVNeed:
             raise ValueError(f"a cache of {self.kv_heads} heads with keys of {self.k_dim} and values of {self.v_dim}")
         if self.key_chunk < 0 or (self.key_chunk and self.k_dim % self.key_chunk != 0):
             raise ValueError(f"keys of {self.k_dim} values cannot be stored in chunks of {self.key_chunk}")
+        if self.pooled < 0 or (self.pooled and self.window is not None):
+            raise ValueError("pooled blocks are kept beside pages that stay: no window, a block of at least one position")
+
+    def pool_slots(self, page_size: int) -> int:
+        """Blocks that can end in one page."""
+        return -(-page_size // self.pooled) if self.pooled else 0
 
     def key_page_shape(self, page_size: int) -> Tuple[int, ...]:
         """Shape of the keys of one key/value head in one page."""

@@ -5,13 +5,20 @@ S_t = decay_h * S_(t-1) + k_t v_t^T and o_t = S_t^T q_t, with no other scale.  T
 (weight `norm`), multiplied lane by lane with sigmoid(W_g h), and projected by W_o into the residual stream.  S starts at zero,
 is float32 [heads, dim, vdim] for every live request, and is all this mixer keeps: it has no pages, and a prompt may be cut
 anywhere.  q, k, v and the gate are one product with the concatenated matrix.
+
+What a design may choose otherwise: `position` (rotary on the first lanes of every head of q and of k, in float32 behind the
+product, lane i with lane i + dims / 2), `key_scale` (a constant on k behind the rotation), `head_norm` (every head's output
+is divided by its own root mean square, no weight, instead of the weighted norm over all heads) and `gate_activation`
+"silu" (the gate is silu(W_g h) instead of a sigmoid).  With rotation or a key scale the operands of the recurrence are
+float32 in both precisions: nothing that enters the recurrence is rounded behind the projection.
 """
 from __future__ import annotations
 
 import numpy as np
 import torch
 
-from ..registry import register_part
+from ..config.spec import PartSpec
+from ..registry import part_class, register_part
 from .base import INIT_MATRIX, INIT_NORM, Mixer, StateNeed, add_and_prepare
 
 
@@ -46,7 +53,22 @@ class LightningAttention(Mixer):
         self.decay_lo = torch.from_numpy(lo).to(rt.device)
         self.w_qkvg = torch.cat([rt.matrix(weights[n]) for n in ("q", "k", "v", "g")], dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
-        self.norm_weight = rt.vector(weights["norm"])
+        self.head_norm = bool(spec.get("head_norm", False))
+        self.norm_weight = None if self.head_norm else rt.vector(weights["norm"])
+        self.gate_activation = spec.get("gate_activation", "sigmoid")
+        if self.gate_activation not in ("sigmoid", "silu") or (self.gate_activation == "silu" and not self.head_norm):
+            raise ValueError("the gate is a sigmoid, or with `head_norm` a silu")
+        self.key_scale = float(spec.get("key_scale", 1.0))
+        self.position = None
+        position = spec.get("position")
+        if position is not None:
+            position = dict(position)
+            kind = position.pop("kind")
+            self.position = part_class("position", kind)(PartSpec(kind, position), {}, rt)
+            if self.position.pairing != 0 or self.position.dims > self.dim:
+                raise ValueError("linear attention turns lane i with lane i + dims / 2 inside a head")
+        if (self.position is not None or self.key_scale != 1.0) and self.activation != "none":
+            raise ValueError("rotated or scaled operands come without an activation")
         rt.tile_for_decode(self.w_o)
         rt.tile_for_decode(self.w_qkvg, priority=1)
 
@@ -60,10 +82,21 @@ class LightningAttention(Mixer):
         qkvg = rt.empty((rows, 2 * nq + 2 * nv))
         ops.linear(h, self.w_qkvg, qkvg)
         o = rt.empty((rows, nv), torch.float32)
-        ops.linear_attention(qkvg, self.decay_hi, self.decay_lo, binding.state, ctx.row_seg, ctx.seg_start, ctx.slots, o,
+        operands = qkvg
+        if self.position is not None or self.key_scale != 1.0:
+            operands = rt.empty((rows, 2 * nq + nv), torch.float32)
+            if self.position is not None:
+                cos, sin, dims = self.position.cos, self.position.sin, self.position.dims
+            else:
+                cos, sin, dims, _ = ctx.no_rotation(rt)
+            ops.rotate_scale(qkvg, operands, ctx.row_pos, cos, sin, self.heads, self.dim, self.v_dim, dims, self.key_scale)
+        ops.linear_attention(operands, self.decay_hi, self.decay_lo, binding.state, ctx.row_seg, ctx.seg_start, ctx.slots, o,
                              self.heads, self.dim, self.v_dim, activation=self.activation)
         gated = rt.empty((rows, nv))
-        ops.gated_norm(o, self.norm_weight, self.eps, qkvg[:, 2 * nq + nv:], gated)
+        if self.head_norm:
+            ops.group_norm_gate(o, self.eps, self.v_dim, qkvg[:, 2 * nq + nv:], gated, activation=self.gate_activation)
+        else:
+            ops.gated_norm(o, self.norm_weight, self.eps, qkvg[:, 2 * nq + nv:], gated)
         if branch is not None:
             ops.linear(gated, self.w_o, branch)
         elif not add_and_prepare(ctx, ops, gated, self.w_o, residual, None):

@@ -8,6 +8,8 @@ phase = position * inv[l] in float32; cos and sin are evaluated in float64 and s
 cos and sin by a magnitude (rope.rs:70-110); `longrope` divides the frequencies by one of two lists of
 per-lane factors, the long one when the tables reach beyond the original context, and multiplies cos and sin
 by its attention factor (rope.rs:30-36, :58-61).  All of it in float32 up to the phase, as the reference.
+`precise` (plain and `yarn` tables): frequencies and phases are computed in float64 and only cos and sin are rounded to
+float32, for designs whose positions are checked more closely than a float32 product of position and frequency allows.
 """
 from __future__ import annotations
 
@@ -53,7 +55,10 @@ class Rotary(Part):
         if self.dims % 2 != 0 or self.dims <= 0:
             raise ValueError("rotary dims must be even and positive")
         positions = int(min(rt.max_context, spec.get("max_position", rt.max_context)))
-        key = ("rotary", self.dims, self.theta, self.scaling, positions) + tuple(
+        self.precise = bool(spec.get("precise", False))
+        if self.precise and self.scaling not in ("none", "yarn"):
+            raise ValueError("precise tables are built for plain and yarn scaling")
+        key = ("rotary", self.dims, self.theta, self.scaling, positions, self.precise) + tuple(
             tuple(v) if isinstance(v, (list, tuple)) else v
             for v in (spec.get(k) for k in ("factor", "low_freq_factor", "high_freq_factor", "original_max_position",
                                             "extrapolation", "attention", "beta_fast", "beta_slow", "truncate",
@@ -72,6 +77,8 @@ class Rotary(Part):
         # float32 powf of float32 operands, correctly rounded: evaluated in float64, rounded once
         base = torch.tensor(self.theta, dtype=torch.float32).double()
         inv = 1.0 / torch.pow(base, exponent.double()).to(torch.float32)
+        if self.precise:
+            inv = 1.0 / torch.pow(torch.tensor(self.theta, dtype=torch.float64), 2.0 * lanes.double() / float(self.dims))
         if self.scaling == "llama3":
             s = self.spec
             inv = inv / llama3_divisors(self.dims, self.theta, float(s["factor"]), float(s["low_freq_factor"]),
@@ -93,6 +100,8 @@ class Rotary(Part):
         elif self.scaling not in ("none", "llama3"):
             raise ValueError(f"unknown rotary scaling {self.scaling!r}")
         pos = torch.arange(positions, dtype=torch.float32) * scale
+        if self.precise:
+            pos = pos.double()
         phase = (pos[:, None] * inv[None, :]).to(torch.float64)          # float32 product, then widened
         cos, sin = torch.cos(phase).to(torch.float32), torch.sin(phase).to(torch.float32)
         if magnitude is not None:
@@ -103,7 +112,8 @@ class Rotary(Part):
         """rope.rs:70-110, every step in float32 as there.  The lanes below `low` keep their angle, the lanes
         above `high` get the angle of position / factor, the lanes between a mix of both."""
         s = self.spec
-        f32 = lambda v: torch.tensor(float(v), dtype=torch.float32)
+        kind = torch.float64 if self.precise else torch.float32
+        f32 = lambda v: torch.tensor(float(v), dtype=kind)
         half = self.dims // 2
         factor, extrapolation = f32(s["factor"]), f32(s.get("extrapolation", 1.0))
         base, original, dims = f32(self.theta), f32(int(s["original_max_position"])), f32(self.dims)
@@ -120,9 +130,9 @@ class Rotary(Part):
         if s.get("truncate", True):
             low, high = torch.floor(low), torch.ceil(high)
         low, high = torch.clamp(low, min=0.0), torch.clamp(high, max=float(self.dims) - 1.0)
-        lanes = torch.arange(half, dtype=torch.float32)
+        lanes = torch.arange(half, dtype=kind)
         ramp = f32(1.0) - torch.clamp((lanes - low) / torch.clamp(high - low, min=0.001), 0.0, 1.0)   # rope.rs:20-23
-        pos = torch.arange(positions, dtype=torch.float32)
+        pos = torch.arange(positions, dtype=kind)
         extrapolated = pos[:, None] * inv[None, :]
         interpolated = scale * extrapolated
         if float(extrapolation) != 0.0:

@@ -362,6 +362,166 @@ class ReferenceOps:
                 out[r, h * v_dim:(h + 1) * v_dim] = o.to(out.dtype)
         return out
 
+    # ---- attention with normed heads or projections, pooled blocks behind a window, sigmoid weights; retention's operands;
+    # routers with groups; experts without a gate; what a pass of looped layers mixes into the stream ----
+    def normed_rope_store(self, qkv, norm_mode, q_weight, k_weight, eps, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,
+                          heads, kv_heads, k_dim, v_dim, rope_dims, page_size, key_chunk, values_from_keys=False):
+        nq, nk, nv = heads * k_dim, kv_heads * k_dim, kv_heads * v_dim
+        half = rope_dims // 2
+        for r in range(qkv.shape[0]):
+            seg = int(row_seg[r])
+            if seg < 0:
+                continue
+            pos = int(row_pos[r])
+            q, k = qkv[r, :nq].double(), qkv[r, nq:nq + nk].double()
+            raw_k = qkv[r, nq:nq + nk]
+            if norm_mode == 2:        # one mean over the whole projection
+                q = q / torch.sqrt((q * q).mean() + eps) * q_weight.double()
+                k = k / torch.sqrt((k * k).mean() + eps) * k_weight.double()
+            q, k = q.view(heads, k_dim).clone(), k.view(kv_heads, k_dim).clone()
+            if norm_mode == 1:        # a mean a head, one weight vector for all heads
+                q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.double()
+                k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.double()
+            if half:
+                c, s = cos[pos].double(), sin[pos].double()
+                for t in (q, k):
+                    a, b = t[:, :half].clone(), t[:, half:rope_dims].clone()
+                    t[:, :half] = a * c - b * s
+                    t[:, half:rope_dims] = b * c + a * s
+            q_out[r] = q.reshape(-1).to(q_out.dtype)
+            if k_pages is None:
+                continue
+            page, off = int(tables[seg, pos // page_size]), pos % page_size
+            k_pages[page, :, :, off, :] = k.view(kv_heads, k_dim // key_chunk, key_chunk).to(k_pages.dtype)
+            v = raw_k if values_from_keys else qkv[r, nq + nk:nq + nk + nv]
+            v_pages[page, :, :, off] = v.view(kv_heads, v_dim)
+        return q_out
+
+    def pool_blocks(self, k_pages, v_pages, pool_k, pool_v, tables, row_pos, row_seg, kv_heads, k_dim, v_dim, page_size, key_chunk, pool):
+        for r in range(row_pos.shape[0]):
+            seg, pos = int(row_seg[r]), int(row_pos[r])
+            if seg < 0 or (pos + 1) % pool != 0:
+                continue
+            keys = torch.arange(pos - pool + 1, pos + 1)
+            pages, offs = tables[seg, (keys // page_size).long()].long(), (keys % page_size).long()
+            k = k_pages[pages, :, :, offs, :].double().reshape(pool, kv_heads, k_dim).mean(0)
+            v = v_pages[pages, :, :, offs].double().mean(0)
+            page, slot = int(tables[seg, pos // page_size]), (pos % page_size) // pool
+            pool_k[page, :, slot] = k.to(pool_k.dtype)
+            pool_v[page, :, slot] = v.to(pool_v.dtype)
+
+    def pooled_window_attention(self, q, k_pages, v_pages, pool_k, pool_v, tables, row_pos, row_seg, seg_start, out, heads, kv_heads,
+                                k_dim, v_dim, page_size, scale, window, pool, key_chunk, max_context=0):
+        group = heads // kv_heads
+        for r in range(q.shape[0]):
+            seg = int(row_seg[r])
+            if seg < 0:
+                out[r] = 0
+                continue
+            pos = int(row_pos[r])
+            keys = torch.arange(max(0, pos - window + 1), pos + 1)
+            pages, offs = tables[seg, (keys // page_size).long()].long(), (keys % page_size).long()
+            k = k_pages[pages, :, :, offs, :].double().reshape(len(keys), kv_heads, k_dim)
+            v = v_pages[pages, :, :, offs].double()
+            blocks = max(0, (pos - window + 1) // pool)
+            if blocks:
+                ends = torch.arange(blocks) * pool + pool - 1
+                bp, slot = tables[seg, (ends // page_size).long()].long(), ((ends % page_size) // pool).long()
+                k = torch.cat([pool_k[bp, :, slot].double(), k], 0)
+                v = torch.cat([pool_v[bp, :, slot].double(), v], 0)
+            qr = q[r].double().view(heads, k_dim)
+            for h in range(heads):
+                p = torch.softmax((k[:, h // group, :] @ qr[h]) * scale, dim=0)
+                out[r, h * v_dim:(h + 1) * v_dim] = (p @ v[:, h // group, :]).to(out.dtype)
+        return out
+
+    def sigmoid_attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, seg_start, out, heads, kv_heads, k_dim, v_dim, page_size,
+                          scale, softcap, r1, r2, pb, temp_coef, temp_every, key_chunk, max_context=0):
+        group = heads // kv_heads
+        for r in range(q.shape[0]):
+            seg = int(row_seg[r])
+            if seg < 0:
+                out[r] = 0
+                continue
+            pos = int(row_pos[r])
+            keys = torch.arange(0, pos + 1)
+            pages, offs = tables[seg, (keys // page_size).long()].long(), (keys % page_size).long()
+            k = k_pages[pages, :, :, offs, :].double().reshape(len(keys), kv_heads, k_dim)
+            v = v_pages[pages, :, :, offs].double()
+            temp = 1.0 + temp_coef * math.log(math.floor((pos + 1) / temp_every) + 1.0)
+            qr = q[r].double().view(heads, k_dim)
+            for h in range(heads):
+                s = (k[:, h // group, :] @ qr[h]) * (scale * temp)
+                s = softcap * torch.tanh(s / softcap) - r1[h].double() * torch.log1p(r2[h].double() * (pos - keys).double())
+                out[r, h * v_dim:(h + 1) * v_dim] = (torch.sigmoid(s + pb[h].double()) @ v[:, h // group, :]).to(out.dtype)
+        return out
+
+    def rotate_scale(self, qkv, out, row_pos, cos, sin, heads, dim, vdim, rope_dims, key_scale):
+        nq, half = heads * dim, rope_dims // 2
+        for r in range(qkv.shape[0]):
+            pos = int(row_pos[r])
+            q, k = qkv[r, :nq].double().view(heads, dim).clone(), qkv[r, nq:2 * nq].double().view(heads, dim).clone()
+            if half:
+                c, s = cos[pos].double(), sin[pos].double()
+                for t in (q, k):
+                    a, b = t[:, :half].clone(), t[:, half:rope_dims].clone()
+                    t[:, :half] = a * c - b * s
+                    t[:, half:rope_dims] = b * c + a * s
+            out[r, :nq] = q.reshape(-1).to(out.dtype)
+            out[r, nq:2 * nq] = (k * key_scale).reshape(-1).to(out.dtype)
+            out[r, 2 * nq:] = qkv[r, 2 * nq:2 * nq + heads * vdim].to(out.dtype)
+        return out
+
+    def group_norm_gate(self, x, eps, group, gate, out, activation="silu"):
+        rows, width = x.shape
+        v = x.double().view(rows, width // group, group)
+        v = (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).view(rows, width)
+        g = gate.double()
+        g = g / (1.0 + torch.exp(-g)) if activation == "silu" else torch.sigmoid(g)
+        out.copy_((v * g).to(out.dtype))
+        return out
+
+    def route_grouped(self, h, w_router, correction, top, groups, groups_kept, ids, weights, route_scale=1.0):
+        z = (h.double() @ w_router.double().T).float()
+        score = torch.sigmoid(z)
+        choice = score + correction.float()
+        rows, E = choice.shape
+        if groups > 1:
+            per = E // groups
+            best = torch.sort(choice.view(rows, groups, per), dim=-1, descending=True)[0][..., :2].sum(-1)
+            kept = torch.sort(best, dim=1, descending=True, stable=True)[1][:, :groups_kept]
+            allowed = torch.zeros((rows, groups), dtype=torch.bool)
+            allowed.scatter_(1, kept, True)
+            choice = torch.where(allowed.repeat_interleave(per, dim=1), choice, torch.full_like(choice, -math.inf))
+        order = torch.sort(choice, dim=1, descending=True, stable=True)[1][:, :top]
+        ids.copy_(order.to(ids.dtype))
+        picked = torch.gather(score, 1, order)
+        weights.copy_(picked / (picked.sum(1, keepdim=True) + 1e-20) * route_scale)
+        return ids, weights
+
+    def experts_up(self, h, ids, w_up, act, activation="relu2"):
+        rows, top = ids.shape
+        for r in range(rows):
+            for k in range(top):
+                y = w_up[int(ids[r, k])].double() @ h[r].double()
+                act[r * top + k] = (torch.clamp(y, min=0.0) ** 2).to(act.dtype)
+        return act
+
+    def activation(self, x, out, kind="relu2"):
+        out.copy_((torch.clamp(x.double(), min=0.0) ** 2).to(out.dtype))
+        return out
+
+    def stream_concat(self, x, ids, table, scale, out):
+        width = x.shape[1]
+        out[:, :width] = x.to(out.dtype)
+        out[:, width:] = (table[ids.long()].double() * scale).to(out.dtype)
+        return out
+
+    def weighted_sum(self, out, x, a, y, b, accumulate=False):
+        v = a * x.double() + b * y.double()
+        out.copy_(((out.double() + v) if accumulate else v).to(out.dtype))
+        return out
+
     def carry_ids(self, ids, source, previous):
         for r in range(ids.numel()):
             if int(source[r]) >= 0:
