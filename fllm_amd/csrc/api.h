@@ -370,6 +370,56 @@ int fllm_head_norm_kv_store(void *qkv, int ld, float eps, int norm_dim, const in
                             const int32_t *tables, int table_stride, void *k_pages, void *v_pages, int rows, int heads, int kv_heads,
                             int head_dim, int v_dim, int page_size, int key_chunk, int dtype, int store_kv, hipStream_t stream);
 
+// ---- mixers beside the softmax attention over all keys (mixer_variants.hip) ----
+// Rows of a joint product [q | k | v | ..]: norm_mode 0 none, 1 an RMS norm of every head of q and of k over its own lanes with
+// one weight vector [k_dim] for all heads, 2 an RMS norm over the whole query projection and over the whole key projection
+// with weights of those sizes; rotary on the first rope_dims lanes of every head (lane i with lane i + rope_dims / 2);
+// queries to q_out, keys and values into the pages.  values_from_keys: the values are the keys as projected and the rows
+// hold no value columns.
+int fllm_normed_rope_store(const void *qkv, int ld, int norm_mode, const float *q_weight, const float *k_weight, float eps, void *q_out,
+                           const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables, int table_stride,
+                           const float *cos_table, const float *sin_table, int table_positions, void *k_pages, void *v_pages, int rows,
+                           int heads, int kv_heads, int k_dim, int v_dim, int rope_dims, int page_size, int key_chunk, int dtype,
+                           int store_kv, int values_from_keys, hipStream_t stream);
+// For every row whose position ends a block of `pool` positions: the float32 means of the block's keys and values, read from
+// the pages, into pool_k / pool_v [page][kv_head][ceil(page_size / pool)][k_dim or v_dim] at the page of the block's last token,
+// slot (that token's place in the page) / pool.
+int fllm_pool_blocks(const void *k_pages, const void *v_pages, float *pool_k, float *pool_v, const int32_t *tables, int table_stride,
+                     const int32_t *row_pos, const int32_t *row_seg, int rows, int kv_heads, int k_dim, int v_dim, int page_size,
+                     int key_chunk, int pool, int dtype, hipStream_t stream);
+// A row at position p sees the tokens max(0, p - window + 1) .. p and one mean key and value for every block b of `pool`
+// positions with b * pool + pool - 1 <= p - window; one softmax over both.
+int fllm_pooled_window_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const float *pool_k,
+                                 const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
+                                 const int32_t *row_seg, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim,
+                                 int page_size, float scale, int window, int pool, int key_chunk, int dtype, hipStream_t stream);
+// out[h] = sum over the keys j <= p of sigmoid(cap * tanh(s / cap) - r1[h] * ln(1 + r2[h] * (p - j)) + pb[h]) * v_j with
+// s = q . k_j * scale * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)).
+int fllm_sigmoid_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables, int table_stride,
+                           const int32_t *row_pos, const int32_t *row_seg, void *out, int rows, int heads, int kv_heads, int head_dim,
+                           int v_dim, int page_size, float scale, float softcap, const float *r1, const float *r2, const float *pb,
+                           float temp_coef, int temp_every, int key_chunk, int dtype, hipStream_t stream);
+// Rows [q | k | v | ..] (heads * dim, heads * dim, heads * vdim) -> float32 rows [q | k | v]: q and k rotated on the first
+// rope_dims lanes of every head at the row's position, k times key_scale, v as it is.
+int fllm_rotate_scale(const void *qkv, int ld, float *out, const int32_t *row_pos, const float *cos_table, const float *sin_table,
+                      int table_positions, int rows, int heads, int dim, int vdim, int rope_dims, float key_scale, int dtype,
+                      hipStream_t stream);
+// out = x / rms(x over each group of `group` lanes) * act(gate), act silu or sigmoid; x float32 or of `dtype`.
+int fllm_group_norm_gate(const void *x, int x_dtype, float eps, int group, const void *gate, int gate_ld, void *out, int rows, int width,
+                         int silu, int dtype, hipStream_t stream);
+// out = a x + b y (accumulate: out += a x + b y), float32.
+int fllm_weighted_sum(float *out, const float *x, float a, const float *y, float b, size_t total, int accumulate, hipStream_t stream);
+// out[r] = [x[r] | table[ids[r]] * scale] in `dtype` (x float32, table of `dtype`), rows of 2 * width.
+int fllm_stream_concat(const float *x, const int32_t *ids, const void *table, int vocab, float scale, void *out, int rows, int width,
+                       int dtype, hipStream_t stream);
+// out = relu(x)^2, element by element (out may be x).
+int fllm_relu_squared(const void *x, void *out, size_t total, int dtype, hipStream_t stream);
+// Router with corrections and groups, and the up product of experts without a gate (routed_experts.hip).
+int fllm_route_grouped(const void *h, int ldh, const void *w_router, const float *correction, int rows, int K, int E, int top, int groups,
+                       int kept, int32_t *ids, float *weights, float route_scale, int dtype, hipStream_t stream);
+int fllm_experts_up(const void *h, int ldh, const int32_t *ids, int rows, int top, const void *w_up, int E, int inter, int K, void *act,
+                    int dtype, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

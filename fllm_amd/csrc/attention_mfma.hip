@@ -591,6 +591,7 @@ attn_tile32_kernel(AttnArgs p) {
                     o[db][j] = fmaf(__hip_atomic_load(from + (db * 16 + j) * THREADS + threadIdx.x, __ATOMIC_RELAXED,
                                                       __HIP_MEMORY_SCOPE_AGENT), f, o[db][j]);
         }
+        m_run = m_all;      // the sum now stands against the maximum of all parts: a sink's term must be scaled to that one
     }
     if (rvalid) {
         l_run = with_sink(l_run, m_run * sc, p.sinks, head);      // the maximum is in raw units here

@@ -118,11 +118,112 @@ route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, i
         weights[r * top + k] = (renormalize || route_scale != 1.0f) ? picks[k] * factor : picks[k];
 }
 
+// Router with corrections and groups: score = sigmoid(W h); the picks are made by choice = score + correction, and only among
+// the experts of the `kept` groups (of `groups` equal groups of neighbours) whose two largest choices sum highest, the lower
+// group among equals; weights[r, k] = the plain score of pick k divided by the sum of the picks' scores (+ 1e-20), times
+// route_scale.  One workgroup a row; one wave chooses.
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+route_grouped_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, const float *__restrict__ correction, int K, int E,
+                     int top, int groups, int kept, int32_t *__restrict__ ids, float *__restrict__ weights, float route_scale) {
+    extern __shared__ float smem[];
+    float *xs = smem;            // K
+    float *score = smem + K;     // E
+    float *choice = score + E;   // E
+    float *gsum = choice + E;    // groups
+    float *picks = gsum + groups;   // top
+    const size_t r = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(h[r * ldh + c]);
+    __syncthreads();
+    const bool vec = sizeof(T) == 2 && K % 8 == 0 && ((uintptr_t)w & 15) == 0;
+    for (int e = wave; e < E; e += kWaves) {
+        const float z = row_dot<T>(xs, w + (size_t)e * K, K, lane, vec);
+        if (lane == 0) {
+            const float s = 1.0f / (1.0f + expf(-z));
+            score[e] = s;
+            choice[e] = s + correction[e];
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const int per = E / groups;
+    if (groups > 1) {
+        for (int g = lane; g < groups; g += kWave) {      // a group counts the sum of its two largest choices (of its one, if it has one)
+            float a = -INFINITY, b = -INFINITY;
+            for (int e = g * per; e < (g + 1) * per; e++) {
+                const float c = choice[e];
+                if (c > a) b = a, a = c;
+                else if (c > b) b = c;
+            }
+            gsum[g] = per > 1 ? a + b : a;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+        for (int k = 0; k < kept; k++) {                  // the best group not yet kept: marked with +inf
+            float best = -INFINITY;
+            int at = 0x7fffffff;
+            for (int g = lane; g < groups; g += kWave) {
+                const float s = gsum[g];
+                if (s != INFINITY && s > best) best = s, at = g;
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float other = __shfl_xor(best, o, kWave);
+                const int other_at = __shfl_xor(at, o, kWave);
+                if (other > best || (other == best && other_at < at)) best = other, at = other_at;
+            }
+            if (at < 0 || at >= groups) {                 // sums that compare with nothing: the first group not yet kept
+                at = 0;
+                while (at < groups - 1 && gsum[at] == INFINITY) at++;
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (lane == 0) gsum[at] = INFINITY;
+            __builtin_amdgcn_wave_barrier();
+            __threadfence_block();
+        }
+        for (int e = lane; e < E; e += kWave)
+            if (gsum[e / per] != INFINITY) choice[e] = -INFINITY;
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    float picked = 0.f;
+    for (int k = 0; k < top; k++) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane; e < E; e += kWave) {
+            const float s = choice[e];
+            if (s > best) best = s, at = e;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float other = __shfl_xor(best, o, kWave);
+            const int other_at = __shfl_xor(at, o, kWave);
+            if (other > best || (other == best && other_at < at)) best = other, at = other_at;
+        }
+        if (at < 0 || at >= E) at = k;
+        const float s = score[at];
+        picked += s;
+        __builtin_amdgcn_wave_barrier();
+        if (lane == 0) {
+            ids[r * top + k] = at;
+            picks[k] = s;
+            choice[at] = -INFINITY;
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+    const float factor = route_scale / (picked + 1e-20f);
+    for (int k = lane; k < top; k += kWave) weights[r * top + k] = picks[k] * factor;
+}
+
 // One (row, pick) pair a workgroup row (blockIdx.y), kCols output columns a workgroup (blockIdx.x), two a wave.
 // MODE 0: act[pair, c] = a(g) * (u + up_offset) with g, u = W_gate[e] x, W_up[e] x (clamped to `limit` when > 0),
 //         a(g) = g * sigmoid(alpha g), x = the row times the pick's weight (rounded to the element type, as a stored
 //         operand would be); w = [E][2 I][K], gate rows then up rows.
 // MODE 1: out[pair, c] = W[e][c] . x, float32; w = [E][N][K]; x = act[pair].
+// MODE 2: act[pair, c] = relu(W[e][c] . x)^2 with x = the pair's row as it is (an expert without a gate, its weight waits for
+//         the output); w = [E][N][K].
 constexpr int kColsPerWave = 2;
 constexpr int kCols = kWaves * kColsPerWave;
 
@@ -140,6 +241,9 @@ expert_rows_kernel(const T *__restrict__ x, int ldx, const int32_t *__restrict__
         const float scale = weights[pair];
         const T *src = x + (pair / top) * ldx;
         for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(from_f32<T>(to_f32<T>(src[c]) * scale));
+    } else if (MODE == 2) {
+        const T *src = x + (pair / top) * ldx;
+        for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(src[c]);
     } else {
         const T *src = x + pair * ldx;
         for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(src[c]);
@@ -172,7 +276,10 @@ expert_rows_kernel(const T *__restrict__ x, int ldx, const int32_t *__restrict__
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const float y = wave_sum(acc[j]);
-                    if (lane == 0) out[pair * N + c0 + j] = y;
+                    if (MODE == 2) {
+                        const float a = fmaxf(y, 0.f);
+                        if (lane == 0) act[pair * N + c0 + j] = from_f32<T>(a * a);
+                    } else if (lane == 0) out[pair * N + c0 + j] = y;
                 }
             }
             return;
@@ -193,7 +300,10 @@ expert_rows_kernel(const T *__restrict__ x, int ldx, const int32_t *__restrict__
             if (lane == 0) act[pair * N + c] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + up_offset));
         } else {
             const float y = row_dot<T>(xs, w + ((size_t)e * N + c) * K, K, lane, vec);
-            if (lane == 0) out[pair * N + c] = y;
+            if (MODE == 2) {
+                const float a = fmaxf(y, 0.f);
+                if (lane == 0) act[pair * N + c] = from_f32<T>(a * a);
+            } else if (lane == 0) out[pair * N + c] = y;
         }
     }
 }
@@ -247,6 +357,52 @@ extern "C" int fllm_experts_gate_up(const void *h, int ldh, const int32_t *ids, 
             FLLM_REQUIRE(false, "experts_gate_up: unknown dtype %d", dtype);
     }
     return fllm_check_launch("experts_gate_up");
+}
+
+extern "C" int fllm_route_grouped(const void *h, int ldh, const void *w_router, const float *correction, int rows, int K, int E, int top,
+                                  int groups, int kept, int32_t *ids, float *weights, float route_scale, int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && K > 0 && E > 0 && top > 0 && ldh >= K, "route_grouped: bad sizes");
+    FLLM_REQUIRE(groups > 0 && E % groups == 0 && kept > 0 && kept <= groups && top <= kept * (E / groups),
+                 "route_grouped: %d experts in %d groups, %d kept, %d picked", E, groups, kept, top);
+    FLLM_REQUIRE(h && w_router && correction && ids && weights, "route_grouped: operands missing");
+    const size_t smem = (size_t)(K + 2 * E + groups + top) * sizeof(float);
+    FLLM_REQUIRE(smem <= 64 * 1024, "route_grouped: a width of %d with %d experts does not fit into LDS", K, E);
+    if (rows == 0) return 0;
+    if (dtype == FLLM_F32)
+        hipLaunchKernelGGL(route_grouped_kernel<float>, dim3(rows), dim3(kBlock), smem, stream, (const float *)h, ldh, (const float *)w_router,
+                           correction, K, E, top, groups, kept, ids, weights, route_scale);
+    else if (dtype == FLLM_BF16)
+        hipLaunchKernelGGL(route_grouped_kernel<bf16_t>, dim3(rows), dim3(kBlock), smem, stream, (const bf16_t *)h, ldh,
+                           (const bf16_t *)w_router, correction, K, E, top, groups, kept, ids, weights, route_scale);
+    else
+        FLLM_REQUIRE(false, "route_grouped: unknown dtype %d", dtype);
+    return fllm_check_launch("route_grouped");
+}
+
+extern "C" int fllm_experts_up(const void *h, int ldh, const int32_t *ids, int rows, int top, const void *w_up, int E, int inter, int K,
+                               void *act, int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && top > 0 && E > 0 && inter > 0 && K > 0 && ldh >= K, "experts_up: bad sizes");
+    FLLM_REQUIRE(h && ids && w_up && act, "experts_up: operands missing");
+    FLLM_REQUIRE((size_t)K * sizeof(float) <= 64 * 1024, "experts_up: a width of %d does not fit into LDS", K);
+    const long pairs = (long)rows * top;
+    FLLM_REQUIRE(pairs <= 65535 * 64L, "experts_up: too many rows");
+    if (pairs == 0) return 0;
+    const size_t smem = (size_t)K * sizeof(float);
+    for (long first = 0; first < pairs; first += 65535) {
+        const int count = (int)(pairs - first < 65535 ? pairs - first : 65535);
+        const dim3 grid((inter + kCols - 1) / kCols, count);
+        FLLM_REQUIRE(first % top == 0 || top == 1 || pairs <= 65535, "experts_up: a launch must begin on a row");
+        if (dtype == FLLM_F32)
+            hipLaunchKernelGGL((expert_rows_kernel<float, 2>), grid, dim3(kBlock), smem, stream, (const float *)h + (first / top) * ldh, ldh,
+                               ids + first, nullptr, top, (const float *)w_up, E, inter, K, (float *)act + first * inter, nullptr, 0.f, 0.f, 0.f);
+        else if (dtype == FLLM_BF16)
+            hipLaunchKernelGGL((expert_rows_kernel<bf16_t, 2>), grid, dim3(kBlock), smem, stream, (const bf16_t *)h + (first / top) * ldh, ldh,
+                               ids + first, nullptr, top, (const bf16_t *)w_up, E, inter, K, (bf16_t *)act + first * inter, nullptr, 0.f, 0.f,
+                               0.f);
+        else
+            FLLM_REQUIRE(false, "experts_up: unknown dtype %d", dtype);
+    }
+    return fllm_check_launch("experts_up");
 }
 
 extern "C" int fllm_experts_down(const void *act, const int32_t *ids, int pairs, const void *w_down, int E, int N, int inter, float *out,

@@ -189,4 +189,4 @@ extern "C" double fllm_probe_mfma_bf16(void *sink, int blocks, int iters, hipStr
 }
 
 extern "C" const char *fllm_last_error(void) { return g_error; }
-extern "C" int fllm_abi_version(void) { return 16; }   // 16: fllm_linear_attention takes room for carried states.  15: fllm_linear_attention takes the form (token after token, chunks on the matrix cores).  14: fllm_attention takes sinks; route_topk takes the score's form, postnorm_add weights a part; short_conv, norm_short_conv, linear_attention, gated_norm, polynorm, head_norm_kv_store.  13: fllm_attention and fllm_rope_kv_store take v_dim, chunk and key_chunk; postnorm_add, route_topk, experts_* (plain and grouped).  12: rmsnorm_pair, glu_clamped, scale_f32, stream_add, qk_norm_rope_store, talking_attention.  11: fllm_linear_f32_tiled.  10: fllm_logprobs_processed, fllm_prepare_norm.  9: tiles for 17 to 64 rows, fllm_scaled_* take w_tiles.  8: weight tiles.  7: fllm_random_fill.  2: fllm_attention takes single_from; probes.  3: fllm_sample takes kinds.  4: fllm_logprobs.  5: FllmAdjustLists.  6: fllm_linear_add_normed, fllm_scaled_*
+extern "C" int fllm_abi_version(void) { return 17; }   // 17: normed_rope_store, pool_blocks, pooled_window_attention, sigmoid_attention, rotate_scale, group_norm_gate, weighted_sum, stream_concat, relu_squared, route_grouped, experts_up.  16: fllm_linear_attention takes room for carried states.  15: fllm_linear_attention takes the form (token after token, chunks on the matrix cores).  14: fllm_attention takes sinks; route_topk takes the score's form, postnorm_add weights a part; short_conv, norm_short_conv, linear_attention, gated_norm, polynorm, head_norm_kv_store.  13: fllm_attention and fllm_rope_kv_store take v_dim, chunk and key_chunk; postnorm_add, route_topk, experts_* (plain and grouped).  12: rmsnorm_pair, glu_clamped, scale_f32, stream_add, qk_norm_rope_store, talking_attention.  11: fllm_linear_f32_tiled.  10: fllm_logprobs_processed, fllm_prepare_norm.  9: tiles for 17 to 64 rows, fllm_scaled_* take w_tiles.  8: weight tiles.  7: fllm_random_fill.  2: fllm_attention takes single_from; probes.  3: fllm_sample takes kinds.  4: fllm_logprobs.  5: FllmAdjustLists.  6: fllm_linear_add_normed, fllm_scaled_*

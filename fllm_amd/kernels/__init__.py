@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 
 def load_library(build_if_missing: bool = True):
@@ -135,6 +135,24 @@ def load_library(build_if_missing: bool = True):
         "fllm_talking_attention": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void,
                                    c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
                                    c_int, c_void, ctypes.c_size_t, c_int, c_void],
+        "fllm_normed_rope_store": [c_void, c_int, c_int, c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_int, c_void, c_void,
+                                   c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                   c_void],
+        "fllm_pool_blocks": [c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int,
+                             c_int, c_int, c_void],
+        "fllm_pooled_window_attention": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int,
+                                         c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void],
+        "fllm_sigmoid_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int,
+                                   c_int, c_int, c_float, c_float, c_void, c_void, c_void, c_float, c_int, c_int, c_int, c_void],
+        "fllm_rotate_scale": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
+                              c_void],
+        "fllm_group_norm_gate": [c_void, c_int, c_float, c_int, c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void],
+        "fllm_weighted_sum": [c_void, c_void, c_float, c_void, c_float, c_size, c_int, c_void],
+        "fllm_stream_concat": [c_void, c_void, c_void, c_int, c_float, c_void, c_int, c_int, c_int, c_void],
+        "fllm_relu_squared": [c_void, c_void, c_size, c_int, c_void],
+        "fllm_route_grouped": [c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void, c_float, c_int,
+                               c_void],
+        "fllm_experts_up": [c_void, c_int, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_void, c_int, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -1131,6 +1149,207 @@ class Ops:
             v_dim, page_size, float(scale), int(chunk) if chunk else 0, key_chunk, _DTYPE_CODE[q.dtype], int(max_context),
             int(splits), _ptr(workspace), ws_floats, 1 if single_rows and rows == seg_start.numel() - 1 else 0, self._stream()))
         return out
+
+    # ---- mixers beside the softmax attention over all keys ----------------------------------------------------------------
+    def _paged(self, q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, k_dim, v_dim, page_size, key_chunk):
+        rows = q.shape[0]
+        _need(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == heads * k_dim and q.dtype in _DTYPE_CODE,
+              f"q must be [rows, {heads * k_dim}] of float32 or bfloat16 with unit column stride")
+        _need(heads % kv_heads == 0, f"{heads} heads are not a multiple of {kv_heads} key/value heads")
+        self._talking_pages(k_pages, v_pages, q.dtype, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(out, "out", q.dtype, (rows, heads * v_dim))
+        return rows, (q.stride(0) if rows > 1 else heads * k_dim)
+
+    def normed_rope_store(self, qkv: torch.Tensor, norm_mode: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                          eps: float, q_out: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, tables: torch.Tensor,
+                          cos: torch.Tensor, sin: torch.Tensor, k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
+                          heads: int, kv_heads: int, k_dim: int, v_dim: int, rope_dims: int, page_size: int, key_chunk: int,
+                          values_from_keys: bool = False) -> torch.Tensor:
+        """Rows of a joint product [q | k | v | ...]: `norm_mode` 0 none, 1 an RMS norm of every head of q and of k with one weight
+        vector [k_dim] for all heads, 2 an RMS norm over the whole query projection and the whole key projection; rotary on the
+        first `rope_dims` lanes of every head (lane i with lane i + rope_dims / 2); queries to `q_out`, keys and values into the
+        pages (None: nothing is stored).  `values_from_keys`: the values are the keys as projected; the rows hold no values."""
+        rows = qkv.shape[0]
+        _need(qkv.is_cuda and qkv.dim() == 2 and qkv.is_contiguous() and qkv.dtype in _DTYPE_CODE, "qkv must be dense rows on the GPU")
+        _need(norm_mode in (0, 1, 2), f"norm mode {norm_mode} unknown")
+        _need(not values_from_keys or v_dim == k_dim, "keys that double as values have one width")
+        _need(qkv.shape[1] >= heads * k_dim + kv_heads * k_dim + (0 if values_from_keys else kv_heads * v_dim), "qkv rows are too short")
+        if norm_mode:
+            _dense(q_weight, "q_weight", torch.float32, (heads * k_dim if norm_mode == 2 else k_dim,))
+            _dense(k_weight, "k_weight", torch.float32, (kv_heads * k_dim if norm_mode == 2 else k_dim,))
+        _dense(q_out, "q_out", qkv.dtype, (rows, heads * k_dim))
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(cos, "cos", torch.float32)
+        _dense(sin, "sin", torch.float32, tuple(cos.shape))
+        _need(cos.dim() == 2 and cos.shape[1] == rope_dims // 2, f"rotary tables must be [positions, {rope_dims // 2}]")
+        store = k_pages is not None
+        if store:
+            self._talking_pages(k_pages, v_pages, qkv.dtype, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        self._check(self.lib.fllm_normed_rope_store(
+            _ptr(qkv), qkv.shape[1], int(norm_mode), _ptr(q_weight) if norm_mode else None, _ptr(k_weight) if norm_mode else None,
+            float(eps), _ptr(q_out), _ptr(row_pos), _ptr(row_seg), _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), cos.shape[0],
+            _ptr(k_pages), _ptr(v_pages), rows, heads, kv_heads, k_dim, v_dim, rope_dims, page_size, key_chunk, _DTYPE_CODE[qkv.dtype],
+            1 if store else 0, 1 if values_from_keys else 0, self._stream()))
+        return q_out
+
+    def _pools(self, pool_k, pool_v, num_pages, kv_heads, k_dim, v_dim, page_size, pool):
+        slots = -(-page_size // pool)
+        _dense(pool_k, "pool_k", torch.float32, (num_pages, kv_heads, slots, k_dim))
+        _dense(pool_v, "pool_v", torch.float32, (num_pages, kv_heads, slots, v_dim))
+
+    def pool_blocks(self, k_pages: torch.Tensor, v_pages: torch.Tensor, pool_k: torch.Tensor, pool_v: torch.Tensor, tables: torch.Tensor,
+                    row_pos: torch.Tensor, row_seg: torch.Tensor, kv_heads: int, k_dim: int, v_dim: int, page_size: int,
+                    key_chunk: int, pool: int) -> None:
+        """For every row whose position ends a block of `pool` positions: the float32 means of the block's keys and values as the
+        pages hold them, into pool_k / pool_v [pages, kv_heads, ceil(page_size / pool), k_dim or v_dim] at the page of the block's
+        last token, slot (the token's place in the page) // pool.  Runs behind the store of the step's keys."""
+        rows = row_pos.numel()
+        _need(pool > 0, "a block holds at least one position")
+        self._talking_pages(k_pages, v_pages, k_pages.dtype, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        _need(k_pages.dtype in _DTYPE_CODE, f"dtype {k_pages.dtype} unsupported")
+        self._pools(pool_k, pool_v, k_pages.shape[0], kv_heads, k_dim, v_dim, page_size, pool)
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        self._check(self.lib.fllm_pool_blocks(_ptr(k_pages), _ptr(v_pages), _ptr(pool_k), _ptr(pool_v), _ptr(tables), tables.shape[1],
+                                              _ptr(row_pos), _ptr(row_seg), rows, kv_heads, k_dim, v_dim, page_size, key_chunk, int(pool),
+                                              _DTYPE_CODE[k_pages.dtype], self._stream()))
+
+    def pooled_window_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, pool_k: torch.Tensor,
+                                pool_v: torch.Tensor, tables: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor,
+                                seg_start: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, k_dim: int, v_dim: int,
+                                page_size: int, scale: float, window: int, pool: int, key_chunk: int, max_context: int = 0) -> torch.Tensor:
+        """A row at position p attends to the tokens max(0, p - window + 1) .. p and to one mean key and value (`pool_blocks`) for
+        every block b of `pool` positions with b * pool + pool - 1 <= p - window, in one softmax."""
+        rows, q_stride = self._paged(q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        _need(window > 0 and pool > 0, "window and pool must be positive")
+        self._pools(pool_k, pool_v, k_pages.shape[0], kv_heads, k_dim, v_dim, page_size, pool)
+        self._check(self.lib.fllm_pooled_window_attention(
+            _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(pool_k), _ptr(pool_v), _ptr(tables), tables.shape[1], _ptr(row_pos),
+            _ptr(row_seg), _ptr(out), rows, heads, kv_heads, k_dim, v_dim, page_size, float(scale), int(window), int(pool), key_chunk,
+            _DTYPE_CODE[q.dtype], self._stream()))
+        return out
+
+    def sigmoid_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tables: torch.Tensor, row_pos: torch.Tensor,
+                          row_seg: torch.Tensor, seg_start: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, k_dim: int,
+                          v_dim: int, page_size: int, scale: float, softcap: float, r1: torch.Tensor, r2: torch.Tensor, pb: torch.Tensor,
+                          temp_coef: float, temp_every: int, key_chunk: int, max_context: int = 0) -> torch.Tensor:
+        """out[h] = sum over the keys j <= p of sigmoid(softcap * tanh(s / softcap) - r1[h] * ln(1 + r2[h] * (p - j)) + pb[h]) * v_j,
+        s = q . k_j * scale * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)); `q` may be a column slice of a wider matrix."""
+        rows, q_stride = self._paged(q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        for name, t in (("r1", r1), ("r2", r2), ("pb", pb)):
+            _dense(t, name, torch.float32, (heads,))
+        _need(softcap > 0 and temp_every > 0, "softcap and temp_every must be positive")
+        self._check(self.lib.fllm_sigmoid_attention(
+            _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg), _ptr(out), rows,
+            heads, kv_heads, k_dim, v_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2), _ptr(pb), float(temp_coef),
+            int(temp_every), key_chunk, _DTYPE_CODE[q.dtype], self._stream()))
+        return out
+
+    def rotate_scale(self, qkv: torch.Tensor, out: torch.Tensor, row_pos: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, heads: int,
+                     dim: int, vdim: int, rope_dims: int, key_scale: float) -> torch.Tensor:
+        """Rows [q | k | v | ..] (heads * dim, heads * dim, heads * vdim) -> float32 rows [q | k | v]: q and k rotated on the first
+        `rope_dims` lanes of every head at the row's position (lane i with lane i + rope_dims / 2), k times `key_scale`."""
+        rows = qkv.shape[0]
+        _need(qkv.is_cuda and qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.dtype in _DTYPE_CODE, "qkv must be a row-major GPU matrix")
+        _need(qkv.shape[1] >= heads * (2 * dim + vdim), "qkv rows are too short")
+        _dense(out, "out", torch.float32, (rows, heads * (2 * dim + vdim)))
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(cos, "cos", torch.float32)
+        _dense(sin, "sin", torch.float32, tuple(cos.shape))
+        _need(cos.dim() == 2 and cos.shape[1] == rope_dims // 2, f"rotary tables must be [positions, {rope_dims // 2}]")
+        self._check(self.lib.fllm_rotate_scale(_ptr(qkv), qkv.stride(0) if rows > 1 else qkv.shape[1], _ptr(out), _ptr(row_pos), _ptr(cos),
+                                               _ptr(sin), cos.shape[0], rows, heads, dim, vdim, rope_dims, float(key_scale),
+                                               _DTYPE_CODE[qkv.dtype], self._stream()))
+        return out
+
+    def group_norm_gate(self, x: torch.Tensor, eps: float, group: int, gate: torch.Tensor, out: torch.Tensor,
+                        activation: str = "silu") -> torch.Tensor:
+        """out = x / sqrt(mean over each group of `group` lanes of x^2 + eps) * act(gate), act "silu" or "sigmoid"; `gate` may be a
+        column slice of a wider matrix."""
+        rows, width = x.shape
+        _dense(x, "x")
+        _need(activation in ("silu", "sigmoid"), f"activation {activation!r} unknown")
+        _need(x.dtype in _DTYPE_CODE and group > 0 and width % group == 0, f"groups of {group} lanes in rows of {width}")
+        _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and tuple(gate.shape) == (rows, width) and gate.dtype == out.dtype,
+              "gate must be [rows, width] of out's type with unit column stride")
+        _dense(out, "out", None, (rows, width))
+        _need(out.dtype in _DTYPE_CODE and (x.dtype == torch.float32 or x.dtype == out.dtype), "group_norm_gate: x is float32 or of out's type")
+        self._check(self.lib.fllm_group_norm_gate(_ptr(x), _DTYPE_CODE[x.dtype], float(eps), int(group), _ptr(gate),
+                                                  gate.stride(0) if rows > 1 else width, _ptr(out), rows, width,
+                                                  1 if activation == "silu" else 0, _DTYPE_CODE[out.dtype], self._stream()))
+        return out
+
+    def weighted_sum(self, out: torch.Tensor, x: torch.Tensor, a: float, y: torch.Tensor, b: float, accumulate: bool = False) -> torch.Tensor:
+        """out = a * x + b * y, or with `accumulate` out += a * x + b * y; float32."""
+        _dense(out, "out", torch.float32)
+        _dense(x, "x", torch.float32, tuple(out.shape))
+        _dense(y, "y", torch.float32, tuple(out.shape))
+        self._check(self.lib.fllm_weighted_sum(_ptr(out), _ptr(x), float(a), _ptr(y), float(b), out.numel(), 1 if accumulate else 0,
+                                               self._stream()))
+        return out
+
+    def stream_concat(self, x: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, scale: float, out: torch.Tensor) -> torch.Tensor:
+        """out[r] = [x[r] | scale * table[ids[r]]] in the table's type: the float32 stream beside the rows' embeddings."""
+        rows, width = x.shape
+        _dense(x, "x", torch.float32)
+        _dense(ids, "ids", torch.int32, (rows,))
+        _dense(table, "table")
+        _need(table.dtype in _DTYPE_CODE and table.dim() == 2 and table.shape[1] == width, f"table must be [vocab, {width}]")
+        _dense(out, "out", table.dtype, (rows, 2 * width))
+        self._check(self.lib.fllm_stream_concat(_ptr(x), _ptr(ids), _ptr(table), table.shape[0], float(scale), _ptr(out), rows, width,
+                                                _DTYPE_CODE[table.dtype], self._stream()))
+        return out
+
+    def activation(self, x: torch.Tensor, out: torch.Tensor, kind: str = "relu2") -> torch.Tensor:
+        """out = relu(x)^2 element by element (`out` may be `x`)."""
+        _need(kind == "relu2", f"activation {kind!r} unknown")
+        _dense(x, "x")
+        _need(x.dtype in _DTYPE_CODE, f"dtype {x.dtype} unsupported")
+        _dense(out, "out", x.dtype, tuple(x.shape))
+        self._check(self.lib.fllm_relu_squared(_ptr(x), _ptr(out), x.numel(), _DTYPE_CODE[x.dtype], self._stream()))
+        return out
+
+    def route_grouped(self, h: torch.Tensor, w_router: torch.Tensor, correction: torch.Tensor, top: int, groups: int, groups_kept: int,
+                      ids: torch.Tensor, weights: torch.Tensor, route_scale: float = 1.0):
+        """score = sigmoid(h @ w_router.T) in float32; the picks are the `top` largest of score + correction among the experts of
+        the `groups_kept` groups (of `groups` equal groups of neighbours) whose two largest corrected scores sum highest (the lower
+        index among equals, for groups and experts); weights = the picks' plain scores / (their sum + 1e-20) * route_scale."""
+        rows, K = h.shape
+        E = w_router.shape[0]
+        _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _DTYPE_CODE, "h must be a row-major GPU matrix")
+        _dense(w_router, "w_router", h.dtype, (E, K))
+        _dense(correction, "correction", torch.float32, (E,))
+        _need(groups > 0 and E % groups == 0 and 0 < groups_kept <= groups and 0 < top <= groups_kept * (E // groups),
+              f"{E} experts in {groups} groups, {groups_kept} kept, {top} picked")
+        _dense(ids, "ids", torch.int32, (rows, top))
+        _dense(weights, "weights", torch.float32, (rows, top))
+        self._check(self.lib.fllm_route_grouped(_ptr(h), h.stride(0) if rows > 1 else K, _ptr(w_router), _ptr(correction), rows, K, E,
+                                                int(top), int(groups), int(groups_kept), _ptr(ids), _ptr(weights), float(route_scale),
+                                                _DTYPE_CODE[h.dtype], self._stream()))
+        return ids, weights
+
+    def experts_up(self, h: torch.Tensor, ids: torch.Tensor, w_up: torch.Tensor, act: torch.Tensor, activation: str = "relu2") -> torch.Tensor:
+        """act[r * top + k] = relu(w_up[ids[r, k]] @ h[r])^2: the up product of experts without a gate; w_up [experts, inter, width]."""
+        rows, K = h.shape
+        top = ids.shape[1]
+        E, inter = w_up.shape[0], w_up.shape[1]
+        _need(activation == "relu2", f"activation {activation!r} unknown")
+        _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _DTYPE_CODE, "h must be a row-major GPU matrix")
+        _dense(w_up, "w_up", h.dtype, (E, inter, K))
+        _dense(ids, "ids", torch.int32, (rows, top))
+        _dense(act, "act", h.dtype, (rows * top, inter))
+        self._check(self.lib.fllm_experts_up(_ptr(h), h.stride(0) if rows > 1 else K, _ptr(ids), rows, top, _ptr(w_up), E, inter, K,
+                                             _ptr(act), _DTYPE_CODE[h.dtype], self._stream()))
+        return act
 
     def measured_ceilings(self, read_bytes: int = 4 << 30, repeats: int = 5) -> dict:
         """What the device delivers to kernels that do nothing else: GB/s of a kernel that only reads a buffer much larger
