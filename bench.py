@@ -264,6 +264,32 @@ def venadra_config(size, layers):
     return cfg, layers
 
 
+def dumizen_config(size, layers):
+    """`layers` layers in turn: sigmoid attention over all keys, two of windowed attention (1,024 tokens, blocks of 64 behind
+    them) and a pair of attention (its keys as values, a zero sink, an output gate) beside retention (as many heads of the same
+    size); routed feed-forwards everywhere: two of eight experts of half the dense width without a gate and a shared one of
+    that width, in two groups of which a token picks inside one (a token multiplies as many weights as the dense gated layer
+    has); the middle half of the layers runs twice, every pass entered through a matrix of twice the width."""
+    heads, kv_heads, dim, ff = size["heads"], size["kv_heads"], size["dim"], size["ff"]
+    scaling = {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}
+    base = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
+    sigmoid = dict(base, softcap=50.0, q_temp={"coef": 0.3, "every": 1024})
+    windowed = dict(base, mask={"size": 1024, "pool": 64}, rot={"dims": dim // 2, "base": 500000.0, "scaling": scaling})
+    both = {"left": dict(base, rot={"dims": dim, "base": 1000000.0, "scaling": scaling}), "left_scale": 0.8, "right_scale": 1.1,
+            "right": {"heads": heads, "dim": dim, "vdim": dim, "rot": {"dims": dim, "base": 1000000.0},
+                      "decay": [1.0 - 2.0 ** -(5 + 5 * h / max(1, heads - 1)) for h in range(heads)]}}
+    mlp = {"kind": "moe", "expert": {"ff": ff // DESIGN_TOP}, "shared": {"ff": ff // DESIGN_TOP},
+           "router": {"experts": DESIGN_EXPERTS, "top": DESIGN_TOP, "scale": 2.0, "groups": {"count": 2, "keep": 1}}}
+    kinds = [("attention_2", sigmoid), ("attention", windowed), ("attention", windowed), ("parallel", both)]
+    cfg = {"architecture": "Dumizen", "width": size["width"], "vocab": size["vocab"], "norm": {"eps": 1e-6}, "max_position": 32768,
+           "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(layers)]}
+    start, stop = layers // 4, layers // 4 + max(1, layers // 2)
+    if stop <= layers and layers >= 3:
+        cfg["loop"] = {"start": start, "stop": stop, "times": 2}
+        return cfg, layers + (stop - start)
+    return cfg, layers
+
+
 def llama_config_of(size, layer_runs):
     return {"model_type": "llama", "architectures": ["LlamaForCausalLM"], "num_hidden_layers": layer_runs,
             "hidden_size": size["width"], "num_attention_heads": size["heads"], "num_key_value_heads": size["kv_heads"],
@@ -272,7 +298,7 @@ def llama_config_of(size, layer_runs):
 
 
 def design_run(args):
-    """Prefill and decode throughput of another design (Menitar, Purivik, Venadra) beside Llama at equal sizes (width, heads, head
+    """Prefill and decode throughput of another design (Menitar, Purivik, Venadra, Dumizen) beside Llama at equal sizes (width, heads, head
     size, feed-forward, vocabulary, as many layers as the other has layer runs), random bfloat16 weights, with the device
     time of the kernels of a decode step and of a prefill step of each.  Prints one JSON line of its own."""
     import gc
@@ -281,8 +307,12 @@ def design_run(args):
     from fllm_amd import Engine, SamplingParams
     size = DESIGN_SIZES[args.design_size]
     layers = args.layers or size["layers"]
-    design, layer_runs = {"menitar": menitar_config, "purivik": purivik_config, "venadra": venadra_config}[args.design](size, layers)
-    models = {args.design: (design, size["vocab"]), "llama": (llama_config_of(size, layer_runs), size["vocab"])}
+    design, layer_runs = {"menitar": menitar_config, "purivik": purivik_config, "venadra": venadra_config,
+                          "dumizen": dumizen_config}[args.design](size, layers)
+    models = {args.design: (design, size["vocab"])}
+    if args.design == "dumizen":       # its closest relative (norms behind the parts, routed experts, looped layers) stands beside it too
+        models["purivik"] = (purivik_config(size, layers)[0], size["vocab"])
+    models["llama"] = (llama_config_of(size, layer_runs), size["vocab"])
     batches = sorted({1, args.batch, 64})
     steps, warmup = min(args.steps, 96), args.warmup
     held = args.prompt_len + warmup + steps + decode_slack(max(batches), args.prompt_len)
@@ -382,7 +412,7 @@ def main():
     ap.add_argument("--sampled", action="store_true",
                     help="for profiling the sampling kernels: the decode runs draw with temperature 0.8, top-k 50 and top-p 0.9 under a "
                          "repetition penalty of 1.1 and report 5 log-probabilities a token (the headline run is greedy)")
-    ap.add_argument("--design", choices=["menitar", "purivik", "venadra"], default=None,
+    ap.add_argument("--design", choices=["menitar", "purivik", "venadra", "dumizen"], default=None,
                     help="instead of the headline run: prefill and decode of this design beside Llama at equal sizes, with the kernels' "
                          "device times of both; prints a line of its own")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="1.5b", help="with --design: the layer sizes")

@@ -391,12 +391,14 @@ int fllm_pool_blocks(const void *k_pages, const void *v_pages, float *pool_k, fl
 // positions with b * pool + pool - 1 <= p - window; one softmax over both.
 int fllm_pooled_window_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const float *pool_k,
                                  const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
-                                 const int32_t *row_seg, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim,
-                                 int page_size, float scale, int window, int pool, int key_chunk, int dtype, hipStream_t stream);
+                                 const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows, int heads,
+                                 int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window, int pool, int key_chunk,
+                                 int dtype, hipStream_t stream);
 // out[h] = sum over the keys j <= p of sigmoid(cap * tanh(s / cap) - r1[h] * ln(1 + r2[h] * (p - j)) + pb[h]) * v_j with
 // s = q . k_j * scale * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)).
 int fllm_sigmoid_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables, int table_stride,
-                           const int32_t *row_pos, const int32_t *row_seg, void *out, int rows, int heads, int kv_heads, int head_dim,
+                           const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
+                           int heads, int kv_heads, int head_dim,
                            int v_dim, int page_size, float scale, float softcap, const float *r1, const float *r2, const float *pb,
                            float temp_coef, int temp_every, int key_chunk, int dtype, hipStream_t stream);
 // Rows [q | k | v | ..] (heads * dim, heads * dim, heads * vdim) -> float32 rows [q | k | v]: q and k rotated on the first

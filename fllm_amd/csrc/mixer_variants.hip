@@ -17,6 +17,18 @@
 #include "api.h"
 #include "common.h"
 
+// mixer_variants_mfma.hip; 1: the shape is not one the matrix-core kernels take
+int fllm_pooled_window_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const float *pool_k,
+                                           const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
+                                           const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
+                                           int heads, int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window,
+                                           int pool, hipStream_t stream);
+int fllm_sigmoid_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
+                                     int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
+                                     int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
+                                     float scale, float softcap, const float *r1, const float *r2, const float *pb, float temp_coef,
+                                     int temp_every, hipStream_t stream);
+
 namespace {
 
 constexpr int kBlock = 256;
@@ -482,9 +494,9 @@ extern "C" int fllm_pool_blocks(const void *k_pages, const void *v_pages, float 
 
 extern "C" int fllm_pooled_window_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const float *pool_k,
                                             const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
-                                            const int32_t *row_seg, void *out, int rows, int heads, int kv_heads, int head_dim,
-                                            int v_dim, int page_size, float scale, int window, int pool, int key_chunk, int dtype,
-                                            hipStream_t stream) {
+                                            const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
+                                            int heads, int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window,
+                                            int pool, int key_chunk, int dtype, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && kv_heads > 0 && head_dim > 0 && v_dim > 0 && page_size > 0 && table_stride > 0,
                  "pooled_window_attention: bad sizes");
     FLLM_REQUIRE(window > 0 && pool > 0, "pooled_window_attention: a window of %d tokens, blocks of %d", window, pool);
@@ -494,6 +506,12 @@ extern "C" int fllm_pooled_window_attention(const void *q, int q_stride, const v
     FLLM_REQUIRE(q_stride >= heads * head_dim, "pooled_window_attention: q_stride %d is shorter than heads * head_dim", q_stride);
     FLLM_REQUIRE(q && k_pages && v_pages && pool_k && pool_v && tables && row_pos && row_seg && out, "pooled_window_attention: operands missing");
     if (rows == 0) return 0;
+    if (dtype == FLLM_BF16 && key_chunk == 8) {
+        const int fast = fllm_pooled_window_attention_bf16_fast(q, q_stride, k_pages, v_pages, pool_k, pool_v, tables, table_stride, row_pos,
+                                                                row_seg, seg_start, num_segs, out, rows, heads, kv_heads, head_dim, v_dim,
+                                                                page_size, scale, window, pool, stream);
+        if (fast <= 0) return fast;
+    }
     const int slots = (page_size + pool - 1) / pool, vd_pad = pow2_lanes(v_dim);
     const size_t smem = (size_t)(((head_dim + 1) & ~1) + kBlock + 2 * ((kWaves + 1) / 2)) * sizeof(float) + (size_t)kBlock * (sizeof(long long) + sizeof(int)) +
                         (size_t)kMaxLanes * kBlock * sizeof(float);
@@ -513,7 +531,8 @@ extern "C" int fllm_pooled_window_attention(const void *q, int q_stride, const v
 }
 
 extern "C" int fllm_sigmoid_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
-                                      int table_stride, const int32_t *row_pos, const int32_t *row_seg, void *out, int rows, int heads,
+                                      int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
+                                      int num_segs, void *out, int rows, int heads,
                                       int kv_heads, int head_dim, int v_dim, int page_size, float scale, float softcap, const float *r1,
                                       const float *r2, const float *pb, float temp_coef, int temp_every, int key_chunk, int dtype,
                                       hipStream_t stream) {
@@ -526,6 +545,12 @@ extern "C" int fllm_sigmoid_attention(const void *q, int q_stride, const void *k
     FLLM_REQUIRE(q_stride >= heads * head_dim, "sigmoid_attention: q_stride %d is shorter than heads * head_dim", q_stride);
     FLLM_REQUIRE(q && k_pages && v_pages && tables && row_pos && row_seg && out && r1 && r2 && pb, "sigmoid_attention: operands missing");
     if (rows == 0) return 0;
+    if (dtype == FLLM_BF16 && key_chunk == 8) {
+        const int fast = fllm_sigmoid_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, seg_start,
+                                                          num_segs, out, rows, heads, kv_heads, head_dim, v_dim, page_size, scale, softcap,
+                                                          r1, r2, pb, temp_coef, temp_every, stream);
+        if (fast <= 0) return fast;
+    }
     const int vd_pad = pow2_lanes(v_dim);
     const size_t smem = (size_t)(((head_dim + 1) & ~1) + kBlock) * sizeof(float) + (size_t)kBlock * (sizeof(long long) + sizeof(int)) +
                         (size_t)kMaxLanes * kBlock * sizeof(float);

@@ -140,10 +140,11 @@ def load_library(build_if_missing: bool = True):
                                    c_void],
         "fllm_pool_blocks": [c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int,
                              c_int, c_int, c_void],
-        "fllm_pooled_window_attention": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int,
-                                         c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void],
-        "fllm_sigmoid_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int,
-                                   c_int, c_int, c_float, c_float, c_void, c_void, c_void, c_float, c_int, c_int, c_int, c_void],
+        "fllm_pooled_window_attention": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void,
+                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void],
+        "fllm_sigmoid_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int, c_int,
+                                   c_int, c_int, c_int, c_int, c_float, c_float, c_void, c_void, c_void, c_float, c_int, c_int, c_int,
+                                   c_void],
         "fllm_rotate_scale": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                               c_void],
         "fllm_group_norm_gate": [c_void, c_int, c_float, c_int, c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void],
@@ -1164,6 +1165,11 @@ class Ops:
         _dense(out, "out", q.dtype, (rows, heads * v_dim))
         return rows, (q.stride(0) if rows > 1 else heads * k_dim)
 
+    @staticmethod
+    def _segments(seg_start, tables, rows):
+        _dense(seg_start, "seg_start", torch.int32)
+        _need(seg_start.numel() >= 2 and tables.shape[0] >= seg_start.numel() - 1, "seg_start must hold a segment's first row and the end; tables a row a segment")
+
     def normed_rope_store(self, qkv: torch.Tensor, norm_mode: int, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
                           eps: float, q_out: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, tables: torch.Tensor,
                           cos: torch.Tensor, sin: torch.Tensor, k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor],
@@ -1230,11 +1236,13 @@ class Ops:
         """A row at position p attends to the tokens max(0, p - window + 1) .. p and to one mean key and value (`pool_blocks`) for
         every block b of `pool` positions with b * pool + pool - 1 <= p - window, in one softmax."""
         rows, q_stride = self._paged(q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        self._segments(seg_start, tables, rows)
         _need(window > 0 and pool > 0, "window and pool must be positive")
         self._pools(pool_k, pool_v, k_pages.shape[0], kv_heads, k_dim, v_dim, page_size, pool)
         self._check(self.lib.fllm_pooled_window_attention(
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(pool_k), _ptr(pool_v), _ptr(tables), tables.shape[1], _ptr(row_pos),
-            _ptr(row_seg), _ptr(out), rows, heads, kv_heads, k_dim, v_dim, page_size, float(scale), int(window), int(pool), key_chunk,
+            _ptr(row_seg), _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, k_dim, v_dim, page_size,
+            float(scale), int(window), int(pool), key_chunk,
             _DTYPE_CODE[q.dtype], self._stream()))
         return out
 
@@ -1245,12 +1253,13 @@ class Ops:
         """out[h] = sum over the keys j <= p of sigmoid(softcap * tanh(s / softcap) - r1[h] * ln(1 + r2[h] * (p - j)) + pb[h]) * v_j,
         s = q . k_j * scale * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)); `q` may be a column slice of a wider matrix."""
         rows, q_stride = self._paged(q, k_pages, v_pages, tables, row_pos, row_seg, out, heads, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        self._segments(seg_start, tables, rows)
         for name, t in (("r1", r1), ("r2", r2), ("pb", pb)):
             _dense(t, name, torch.float32, (heads,))
         _need(softcap > 0 and temp_every > 0, "softcap and temp_every must be positive")
         self._check(self.lib.fllm_sigmoid_attention(
-            _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg), _ptr(out), rows,
-            heads, kv_heads, k_dim, v_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2), _ptr(pb), float(temp_coef),
+            _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg), _ptr(seg_start),
+            seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, k_dim, v_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2), _ptr(pb), float(temp_coef),
             int(temp_every), key_chunk, _DTYPE_CODE[q.dtype], self._stream()))
         return out
 

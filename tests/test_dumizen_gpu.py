@@ -83,7 +83,8 @@ class Scene:
         return out
 
 
-SEGMENTS = [(0, 9), (37, 1), (100, 30), (61, 3), (250, 1)]
+SEGMENTS = [(0, 9), (37, 1), (100, 30), (61, 3), (250, 1), (300, 70)]
+SINGLE_ROWS = [(0, 1), (37, 1), (100, 1), (63, 1), (250, 1), (64, 1), (1000, 1)]
 
 
 # ---------------------------------------------------------------------------------------------
@@ -137,11 +138,18 @@ def fill_pools(ref, sc, t, G, d, dv, pool):
                             torch.full((len(ends),), s, dtype=torch.int32), G, d, dv, sc.page, sc.key_chunk, pool)
 
 
+@pytest.mark.parametrize("rows", ["mixed", "single"])
+@pytest.mark.parametrize("fast", [True, False])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,dv,page,window,pool", [(4, 1, 32, 16, 8, 12, 4), (3, 3, 32, 32, 16, 5, 1), (3, 1, 12, 10, 16, 7, 3),
-                                                         (8, 2, 64, 32, 16, 40, 8), (2, 1, 128, 300, 32, 33, 16)])
-def test_windows_with_pooled_blocks_over_pages(ops, ref, H, G, d, dv, page, window, pool, dtype):
-    sc = Scene(SEGMENTS, G, d, dv, page, seed=d + window, pool=pool)
+                                                         (8, 2, 64, 32, 16, 40, 8), (2, 1, 128, 300, 32, 33, 16), (12, 2, 128, 128, 16, 100, 8),
+                                                         (6, 2, 96, 32, 32, 40, 8)])
+def test_windows_with_pooled_blocks_over_pages(ops, ref, H, G, d, dv, page, window, pool, dtype, fast, rows):
+    """`fast` False: the plain kernel also where the matrix-core kernel would serve (bfloat16, heads of 32 to 128 lanes in
+    steps of 32, pages of multiples of 16); "single": a step of one row a request, whose tiles are the heads of a key/value head."""
+    if dtype == torch.float32 and not fast:
+        pytest.skip("float32 has one kernel")
+    sc = Scene(SINGLE_ROWS if rows == "single" else SEGMENTS, G, d, dv, page, seed=d + window, pool=pool)
     q = torch.randn(sc.rows, H * d, generator=gen(3)).to(dtype).float()
     want_t = sc.to("cpu", torch.float64)
     want_t["k_pages"], want_t["v_pages"] = want_t["k_pages"].to(dtype).double(), want_t["v_pages"].to(dtype).double()
@@ -149,7 +157,12 @@ def test_windows_with_pooled_blocks_over_pages(ops, ref, H, G, d, dv, page, wind
     got_t = sc.to(DEV, dtype)
     got_t["pool_k"], got_t["pool_v"] = want_t["pool_k"].float().to(DEV), want_t["pool_v"].float().to(DEV)
     want = pooled_attend(ref, want_t, q.double(), sc, H, G, d, dv, 0.3, window, pool, torch.float64)
-    got = pooled_attend(ops, got_t, q.to(DEV, dtype), sc, H, G, d, dv, 0.3, window, pool, dtype)
+    ops.set_fast_kernels(fast)
+    try:
+        got = pooled_attend(ops, got_t, q.to(DEV, dtype), sc, H, G, d, dv, 0.3, window, pool, dtype)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_fast_kernels(True)
     close(got_t["pool_k"], want_t["pool_k"], 1e-6, 1e-6, "means of keys")
     close(got_t["pool_v"], want_t["pool_v"], 1e-6, 1e-6, "means of values")
     close(got, want, *((2e-5, 2e-5) if dtype == torch.float32 else (2 * BF16_EPS, 5e-3)), "attention")
@@ -188,10 +201,15 @@ def test_one_key_that_stands_out_at_the_edges(ops, ref, where, held, dtype):
 # ---------------------------------------------------------------------------------------------
 # sigmoid weights
 # ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("rows", ["mixed", "single"])
+@pytest.mark.parametrize("fast", [True, False])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,dv,page", [(4, 2, 16, 24, 8), (3, 3, 32, 32, 16), (3, 1, 12, 20, 16), (4, 2, 64, 64, 16), (2, 1, 96, 300, 32)])
-def test_sigmoid_attention_over_pages(ops, ref, H, G, d, dv, page, dtype):
-    sc = Scene(SEGMENTS, G, d, dv, page, seed=d + dv)
+@pytest.mark.parametrize("H,G,d,dv,page", [(4, 2, 16, 24, 8), (3, 3, 32, 32, 16), (3, 1, 12, 20, 16), (4, 2, 64, 64, 16), (2, 1, 96, 300, 32),
+                                           (12, 2, 128, 128, 16), (4, 2, 96, 96, 32)])
+def test_sigmoid_attention_over_pages(ops, ref, H, G, d, dv, page, dtype, fast, rows):
+    if dtype == torch.float32 and not fast:
+        pytest.skip("float32 has one kernel")
+    sc = Scene(SINGLE_ROWS if rows == "single" else SEGMENTS, G, d, dv, page, seed=d + dv)
     g = gen(4)
     q = torch.randn(sc.rows, H * d + 16, generator=g).to(dtype).float()
     r1, r2, pb = torch.rand(H, generator=g) + 0.2, torch.rand(H, generator=g) * 0.5 + 0.05, torch.randn(H, generator=g) - 1.0
@@ -201,8 +219,16 @@ def test_sigmoid_attention_over_pages(ops, ref, H, G, d, dv, page, dtype):
         if kind == torch.float64:
             t["k_pages"], t["v_pages"] = t["k_pages"].to(dtype).double(), t["v_pages"].to(dtype).double()
         out = torch.empty(sc.rows, H * dv, dtype=kind, device=dev)
-        o.sigmoid_attention(q.to(dev, kind)[:, :H * d], t["k_pages"], t["v_pages"], t["tables"], t["row_pos"], t["row_seg"], t["seg_start"],
-                            out, H, G, d, dv, page, 0.2, 4.0, r1.to(dev), r2.to(dev), pb.to(dev), 0.4, 8, sc.key_chunk, max_context=sc.max_pos)
+        if o is ops:
+            ops.set_fast_kernels(fast)
+        try:
+            o.sigmoid_attention(q.to(dev, kind)[:, :H * d], t["k_pages"], t["v_pages"], t["tables"], t["row_pos"], t["row_seg"], t["seg_start"],
+                                out, H, G, d, dv, page, 0.2, 4.0, r1.to(dev), r2.to(dev), pb.to(dev), 0.4, 8, sc.key_chunk, max_context=sc.max_pos)
+            if o is ops:
+                torch.cuda.synchronize()
+        finally:
+            if o is ops:
+                ops.set_fast_kernels(True)
         outs.append(out)
     scale = outs[0].abs().max().item()
     close(outs[1], outs[0], *((2e-5, 2e-5 * scale) if dtype == torch.float32 else (2 * BF16_EPS, 4e-3 * scale)), "sigmoid attention")
