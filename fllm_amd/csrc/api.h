@@ -393,14 +393,15 @@ int fllm_pooled_window_attention(const void *q, int q_stride, const void *k_page
                                  const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
                                  const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows, int heads,
                                  int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window, int pool, int key_chunk,
-                                 int dtype, hipStream_t stream);
+                                 int dtype, int max_context, hipStream_t stream);
 // out[h] = sum over the keys j <= p of sigmoid(cap * tanh(s / cap) - r1[h] * ln(1 + r2[h] * (p - j)) + pb[h]) * v_j with
-// s = q . k_j * scale * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)).
+// s = q . k_j * scale * (1 + temp_coef * ln(floor((p + 1) / temp_every) + 1)).  max_context bounds position + 1 over the rows (0:
+// unknown); steps of single rows with long contexts share a row's keys among workgroups by it.
 int fllm_sigmoid_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables, int table_stride,
                            const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
                            int heads, int kv_heads, int head_dim,
                            int v_dim, int page_size, float scale, float softcap, const float *r1, const float *r2, const float *pb,
-                           float temp_coef, int temp_every, int key_chunk, int dtype, hipStream_t stream);
+                           float temp_coef, int temp_every, int key_chunk, int dtype, int max_context, hipStream_t stream);
 // Rows [q | k | v | ..] (heads * dim, heads * dim, heads * vdim) -> float32 rows [q | k | v]: q and k rotated on the first
 // rope_dims lanes of every head at the row's position, k times key_scale, v as it is.
 int fllm_rotate_scale(const void *qkv, int ld, float *out, const int32_t *row_pos, const float *cos_table, const float *sin_table,
@@ -421,6 +422,11 @@ int fllm_route_grouped(const void *h, int ldh, const void *w_router, const float
                        int kept, int32_t *ids, float *weights, float route_scale, int dtype, hipStream_t stream);
 int fllm_experts_up(const void *h, int ldh, const int32_t *ids, int rows, int top, const void *w_up, int E, int inter, int K, void *act,
                     int dtype, hipStream_t stream);
+// Experts without a gate on the matrix cores: pairs grouped by expert, act = relu(W_up[e] h)^2, out = W_down[e] act (float32
+// [rows * top, N]); scratch as for fllm_experts_grouped (no scaled rows).  1: shape declined.
+int fllm_experts_grouped_ungated(const void *h, int ldh, const int32_t *ids, int rows, int top, const void *w_up, const void *w_down,
+                                 int E, int inter, int K, int N, void *act, float *out, int32_t *work, float *planes,
+                                 hipStream_t stream);
 
 #ifdef __cplusplus
 }

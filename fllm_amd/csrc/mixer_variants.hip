@@ -22,12 +22,12 @@ int fllm_pooled_window_attention_bf16_fast(const void *q, int q_stride, const vo
                                            const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
                                            const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
                                            int heads, int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window,
-                                           int pool, hipStream_t stream);
+                                           int pool, int max_context, hipStream_t stream);
 int fllm_sigmoid_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                                      int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                                      int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
                                      float scale, float softcap, const float *r1, const float *r2, const float *pb, float temp_coef,
-                                     int temp_every, hipStream_t stream);
+                                     int temp_every, int max_context, hipStream_t stream);
 
 namespace {
 
@@ -126,6 +126,7 @@ pool_blocks_kernel(const T *__restrict__ k_pages, const T *__restrict__ v_pages,
     const size_t dst = (((size_t)tbl[pos / page_size] * kv_heads + kvh) * slots + (pos % page_size) / pool);
     for (int c = threadIdx.x; c < k_dim + v_dim; c += kBlock) {
         float sum = 0.f;
+#pragma unroll 8      // eight loads on their way at once
         for (int t = 0; t < pool; t++) {
             const int key = first + t, page = tbl[key / page_size], off = key % page_size;
             sum += c < k_dim ? to_f32<T>(k_pages[key_at(page, kv_heads, kvh, page_size, k_dim, off, c, key_chunk)])
@@ -496,7 +497,7 @@ extern "C" int fllm_pooled_window_attention(const void *q, int q_stride, const v
                                             const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
                                             const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
                                             int heads, int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window,
-                                            int pool, int key_chunk, int dtype, hipStream_t stream) {
+                                            int pool, int key_chunk, int dtype, int max_context, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && kv_heads > 0 && head_dim > 0 && v_dim > 0 && page_size > 0 && table_stride > 0,
                  "pooled_window_attention: bad sizes");
     FLLM_REQUIRE(window > 0 && pool > 0, "pooled_window_attention: a window of %d tokens, blocks of %d", window, pool);
@@ -509,7 +510,7 @@ extern "C" int fllm_pooled_window_attention(const void *q, int q_stride, const v
     if (dtype == FLLM_BF16 && key_chunk == 8) {
         const int fast = fllm_pooled_window_attention_bf16_fast(q, q_stride, k_pages, v_pages, pool_k, pool_v, tables, table_stride, row_pos,
                                                                 row_seg, seg_start, num_segs, out, rows, heads, kv_heads, head_dim, v_dim,
-                                                                page_size, scale, window, pool, stream);
+                                                                page_size, scale, window, pool, max_context, stream);
         if (fast <= 0) return fast;
     }
     const int slots = (page_size + pool - 1) / pool, vd_pad = pow2_lanes(v_dim);
@@ -535,7 +536,7 @@ extern "C" int fllm_sigmoid_attention(const void *q, int q_stride, const void *k
                                       int num_segs, void *out, int rows, int heads,
                                       int kv_heads, int head_dim, int v_dim, int page_size, float scale, float softcap, const float *r1,
                                       const float *r2, const float *pb, float temp_coef, int temp_every, int key_chunk, int dtype,
-                                      hipStream_t stream) {
+                                      int max_context, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && kv_heads > 0 && head_dim > 0 && v_dim > 0 && page_size > 0 && table_stride > 0,
                  "sigmoid_attention: bad sizes");
     FLLM_REQUIRE(softcap > 0.f && temp_every > 0, "sigmoid_attention: a cap of %g, a temperature step every %d positions", softcap, temp_every);
@@ -548,7 +549,7 @@ extern "C" int fllm_sigmoid_attention(const void *q, int q_stride, const void *k
     if (dtype == FLLM_BF16 && key_chunk == 8) {
         const int fast = fllm_sigmoid_attention_bf16_fast(q, q_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg, seg_start,
                                                           num_segs, out, rows, heads, kv_heads, head_dim, v_dim, page_size, scale, softcap,
-                                                          r1, r2, pb, temp_coef, temp_every, stream);
+                                                          r1, r2, pb, temp_coef, temp_every, max_context, stream);
         if (fast <= 0) return fast;
     }
     const int vd_pad = pow2_lanes(v_dim);

@@ -12,6 +12,8 @@
 //                 in a page (one 16-byte load).
 // Weights stay float32: P goes into the product as the sum of two bfloat16 numbers (its rounding and what the rounding
 // lost), two products a tile.  The means of blocks are float32 in memory and go in the same way, for keys and for values.
+#include <algorithm>
+
 #include "api.h"
 #include "common.h"
 
@@ -37,6 +39,8 @@ struct TileParams {
     int temp_every;
     const float *r1, *r2, *pb;
     int by_heads;                             // 1: a tile is the heads of one key/value head of one row
+    int splits;                               // workgroups that share a tile's keys (blockIdx.z); more than one: partial results
+    float *parts;                             // [tile][split][16 * DV sums, 16 maxima, 16 denominators] for the merge kernel
 };
 
 __device__ __forceinline__ void split_bf16(const float (&x)[8], bf16x8_t &hi, bf16x8_t &lo) {
@@ -66,7 +70,8 @@ mixer_tile_kernel(const TileParams p) {
         head0 = kvh * G;
         count = G;
         if (seg < 0) {      // padding row: zeros
-            for (int i = threadIdx.x; i < G * DV; i += kThreads) p.out[((size_t)row0 * p.heads + head0) * DV + i] = (bf16_t)0.f;
+            if (blockIdx.z == 0)
+                for (int i = threadIdx.x; i < G * DV; i += kThreads) p.out[((size_t)row0 * p.heads + head0) * DV + i] = (bf16_t)0.f;
             return;
         }
     } else {
@@ -172,7 +177,7 @@ mixer_tile_kernel(const TileParams p) {
         const int lo_max = pos_max - p.window + 1 > 0 ? pos_max - p.window + 1 : 0;
         const int nb_max = lo_max / p.pool;
         for (int base = 0; base < nb_max; base += 32, turn++) {
-            if ((turn & (kWavesM - 1)) != wave) continue;
+            if ((turn & (kWavesM - 1)) != wave || (turn / kWavesM) % p.splits != (int)blockIdx.z) continue;
             f32x4_t s[2];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
@@ -222,7 +227,7 @@ mixer_tile_kernel(const TileParams p) {
     {
         const int first = VARIANT == 0 ? (pos_min - p.window + 1 > 0 ? pos_min - p.window + 1 : 0) : 0;
         for (int base = first & ~31; base <= pos_max; base += 32, turn++) {
-            if ((turn & (kWavesM - 1)) != wave) continue;
+            if ((turn & (kWavesM - 1)) != wave || (turn / kWavesM) % p.splits != (int)blockIdx.z) continue;
             f32x4_t s[2];
 #pragma unroll
             for (int j = 0; j < 2; j++) {
@@ -263,6 +268,7 @@ mixer_tile_kernel(const TileParams p) {
 #pragma unroll
         for (int i = 0; i < 4; i++) sm_o[wave][qi][t * 16 + g * 4 + i] = o[t][i];
     __syncthreads();
+    float *part = p.splits > 1 ? p.parts + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * p.splits + blockIdx.z) * (16 * DV + 32) : nullptr;
     for (int idx = threadIdx.x; idx < count * DV; idx += kThreads) {
         const int q = idx / DV, d = idx - q * DV;
         float acc = 0.f, l = 0.f;
@@ -276,13 +282,51 @@ mixer_tile_kernel(const TileParams p) {
                 l += sm_l[w][q] * f;
                 acc += sm_o[w][q][d] * f;
             }
+            if (part != nullptr) {      // this workgroup's share of the keys: the sums as they are, against its own maximum
+                part[q * DV + d] = acc;
+                if (d == 0) part[16 * DV + q] = m, part[16 * DV + 16 + q] = l;
+                continue;
+            }
             acc = l > 0.f ? acc / l : 0.f;
         } else {
 #pragma unroll
             for (int w = 0; w < kWavesM; w++) acc += sm_o[w][q][d];
+            if (part != nullptr) {
+                part[q * DV + d] = acc;
+                continue;
+            }
         }
         const int row = p.by_heads ? row0 : row0 + q, head = p.by_heads ? head0 + q : head0;
         p.out[((size_t)row * p.heads + head) * DV + d] = (bf16_t)acc;
+    }
+}
+
+// The shares of a tile's keys put together in the order of the shares: grid (rows, kv_heads), tiles by heads.
+template <int VARIANT>
+__global__ void __launch_bounds__(kThreads)
+mixer_merge_kernel(const float *__restrict__ parts, int splits, const int32_t *__restrict__ row_seg, bf16_t *__restrict__ out, int heads,
+                   int kv_heads, int DV) {
+    const int row = blockIdx.x, kvh = blockIdx.y, G = heads / kv_heads;
+    if (row_seg[row] < 0) return;
+    const int stride = 16 * DV + 32;
+    const float *mine = parts + (size_t)(blockIdx.y * gridDim.x + blockIdx.x) * splits * stride;
+    for (int idx = threadIdx.x; idx < G * DV; idx += kThreads) {
+        const int q = idx / DV, d = idx - q * DV;
+        float acc = 0.f;
+        if (VARIANT == 0) {
+            float m = -INFINITY, l = 0.f;
+            for (int s = 0; s < splits; s++) m = fmaxf(m, mine[(size_t)s * stride + 16 * DV + q]);
+            for (int s = 0; s < splits; s++) {
+                const float ms = mine[(size_t)s * stride + 16 * DV + q];
+                const float f = ms == -INFINITY ? 0.f : expf(ms - m);
+                l += mine[(size_t)s * stride + 16 * DV + 16 + q] * f;
+                acc += mine[(size_t)s * stride + q * DV + d] * f;
+            }
+            acc = l > 0.f ? acc / l : 0.f;
+        } else {
+            for (int s = 0; s < splits; s++) acc += mine[(size_t)s * stride + q * DV + d];
+        }
+        out[((size_t)row * heads + kvh * G + q) * DV + d] = (bf16_t)acc;
     }
 }
 
@@ -298,22 +342,45 @@ int launch_vt(const TileParams &p, int vt, dim3 grid, hipStream_t stream) {
 }
 
 template <int VARIANT>
-int launch_tiles(TileParams &p, int head_dim, int v_dim, hipStream_t stream) {
+int launch_tiles(TileParams &p, int head_dim, int v_dim, int keys_bound, hipStream_t stream) {
     // takes: bfloat16, keys in chunks of 8 (checked by the caller), heads of 32, 64, 96 or 128 lanes, values of 32, 64, 96 or
     // 128, pages of a multiple of 16 tokens, and for steps of single rows at most 16 heads a key/value head
     if (head_dim % 32 != 0 || head_dim > 128 || v_dim % 32 != 0 || v_dim > 128 || p.page_size % 16 != 0) return 1;
     const int G = p.heads / p.kv_heads;
     p.by_heads = p.rows == p.num_segs ? 1 : 0;
     if (p.by_heads && G > 16) return 1;
-    const dim3 grid = p.by_heads ? dim3(p.rows, p.kv_heads) : dim3((p.rows + 15) / 16 + p.num_segs, p.heads);
+    dim3 grid = p.by_heads ? dim3(p.rows, p.kv_heads) : dim3((p.rows + 15) / 16 + p.num_segs, p.heads);
     if (grid.y > 65535) return 1;
-    switch (head_dim / 32) {
-    case 1: return launch_vt<VARIANT, 1>(p, v_dim / 16, grid, stream);
-    case 2: return launch_vt<VARIANT, 2>(p, v_dim / 16, grid, stream);
-    case 3: return launch_vt<VARIANT, 3>(p, v_dim / 16, grid, stream);
-    case 4: return launch_vt<VARIANT, 4>(p, v_dim / 16, grid, stream);
+    // Steps of single rows have a tile a row and key/value head: with few of them, several workgroups share a tile's keys
+    // (at least 256 keys each, two workgroups a compute unit at most) and a second kernel puts their shares together.
+    p.splits = 1;
+    p.parts = nullptr;
+    if (p.by_heads) {
+        const long tiles = (long)p.rows * p.kv_heads;
+        long splits = std::min<long>(std::min<long>(512 / std::max<long>(tiles, 1), (keys_bound + 255) / 256), 32);
+        void *base = nullptr;
+        size_t bytes = 0;
+        if (splits > 1 && fllm_device_workspace(&base, &bytes) && bytes > kWorkspaceCounterBytes) {
+            const size_t room = (bytes - kWorkspaceCounterBytes) / sizeof(float), each = (size_t)tiles * (16 * v_dim + 32);
+            splits = std::min<long>(splits, (long)(room / each));
+            if (splits > 1) {
+                p.splits = (int)splits;
+                p.parts = (float *)((char *)base + kWorkspaceCounterBytes);
+                grid.z = (unsigned)splits;
+            }
+        }
     }
-    return 1;
+    int declined = 1;
+    switch (head_dim / 32) {
+    case 1: declined = launch_vt<VARIANT, 1>(p, v_dim / 16, grid, stream); break;
+    case 2: declined = launch_vt<VARIANT, 2>(p, v_dim / 16, grid, stream); break;
+    case 3: declined = launch_vt<VARIANT, 3>(p, v_dim / 16, grid, stream); break;
+    case 4: declined = launch_vt<VARIANT, 4>(p, v_dim / 16, grid, stream); break;
+    }
+    if (!declined && p.splits > 1)
+        hipLaunchKernelGGL(mixer_merge_kernel<VARIANT>, dim3(p.rows, p.kv_heads), dim3(kThreads), 0, stream, p.parts, p.splits, p.row_seg, p.out,
+                           p.heads, p.kv_heads, v_dim);
+    return declined;
 }
 
 }  // namespace
@@ -323,14 +390,15 @@ int fllm_pooled_window_attention_bf16_fast(const void *q, int q_stride, const vo
                                            const float *pool_v, const int32_t *tables, int table_stride, const int32_t *row_pos,
                                            const int32_t *row_seg, const int32_t *seg_start, int num_segs, void *out, int rows,
                                            int heads, int kv_heads, int head_dim, int v_dim, int page_size, float scale, int window,
-                                           int pool, hipStream_t stream) {
+                                           int pool, int max_context, hipStream_t stream) {
     if (!fllm_fast_kernels_enabled() || seg_start == nullptr || num_segs <= 0) return 1;
     TileParams p = {};
     p.q = (const bf16_t *)q, p.q_stride = q_stride, p.k_pages = (const bf16_t *)k_pages, p.v_pages = (const bf16_t *)v_pages;
     p.pool_k = pool_k, p.pool_v = pool_v, p.tables = tables, p.table_stride = table_stride, p.row_pos = row_pos, p.row_seg = row_seg;
     p.seg_start = seg_start, p.num_segs = num_segs, p.out = (bf16_t *)out, p.rows = rows, p.heads = heads, p.kv_heads = kv_heads;
     p.page_size = page_size, p.scale = scale, p.window = window, p.pool = pool, p.slots = (page_size + pool - 1) / pool;
-    if (launch_tiles<0>(p, head_dim, v_dim, stream)) return 1;
+    const int span = max_context > 0 ? std::min(max_context, window + (max_context + pool - 1) / pool) : window;
+    if (launch_tiles<0>(p, head_dim, v_dim, span, stream)) return 1;
     return fllm_check_launch("pooled_window_attention (matrix cores)");
 }
 
@@ -338,7 +406,7 @@ int fllm_sigmoid_attention_bf16_fast(const void *q, int q_stride, const void *k_
                                      int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
                                      int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
                                      float scale, float softcap, const float *r1, const float *r2, const float *pb, float temp_coef,
-                                     int temp_every, hipStream_t stream) {
+                                     int temp_every, int max_context, hipStream_t stream) {
     if (!fllm_fast_kernels_enabled() || seg_start == nullptr || num_segs <= 0) return 1;
     TileParams p = {};
     p.q = (const bf16_t *)q, p.q_stride = q_stride, p.k_pages = (const bf16_t *)k_pages, p.v_pages = (const bf16_t *)v_pages;
@@ -346,6 +414,6 @@ int fllm_sigmoid_attention_bf16_fast(const void *q, int q_stride, const void *k_
     p.num_segs = num_segs, p.out = (bf16_t *)out, p.rows = rows, p.heads = heads, p.kv_heads = kv_heads, p.page_size = page_size;
     p.scale = scale, p.softcap = softcap, p.temp_coef = temp_coef, p.temp_every = temp_every, p.r1 = r1, p.r2 = r2, p.pb = pb;
     p.window = 1, p.pool = 1, p.slots = 1;
-    if (launch_tiles<1>(p, head_dim, v_dim, stream)) return 1;
+    if (launch_tiles<1>(p, head_dim, v_dim, max_context, stream)) return 1;
     return fllm_check_launch("sigmoid_attention (matrix cores)");
 }

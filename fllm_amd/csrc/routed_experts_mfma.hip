@@ -84,6 +84,8 @@ scaled_rows_kernel(const bf16_t *__restrict__ h, int ldh, const float *__restric
 // MODE 0: act[pair, c] = a(g) * (u + up_offset) for 64 columns c a workgroup; A rows = the scaled rows in slot order;
 //         B = 64 gate rows and 64 up rows of the expert.  w: [E][2 N][K].
 // MODE 1: out[pair, c] = w[e][c] . act[pair] for GN columns, float32.  w: [E][N][K].
+// MODE 2: act[pair, c] = relu(w[e][c] . h[pair / top])^2 for GN columns: the up product of experts without a gate, whose rows
+//         are read as they are (the picks' weights wait for the outputs).  w: [E][N][K]; x = h, row stride ldx.
 // GN: weight rows a column tile, 128, or 64 (MODE 1 only) where a launch of 128-column tiles would leave most of the
 // device without a workgroup (decode steps).
 // GM: pairs a row tile, 64 (a wave 32 rows) or 128 (a wave 64 rows: an operand read from LDS serves twice the products).
@@ -91,11 +93,11 @@ template <int MODE, int GM, int GN>
 __global__ void __launch_bounds__(kThreads)
 grouped_tiles_kernel(const bf16_t *__restrict__ x, int ldx, const int32_t *__restrict__ work,
                      int max_tiles, const bf16_t *__restrict__ w, int N, int K, bf16_t *__restrict__ act, float *__restrict__ out,
-                     float limit, float alpha, float up_offset, int k_per, size_t slice_stride) {
+                     float limit, float alpha, float up_offset, int k_per, size_t slice_stride, int top) {
     __shared__ __attribute__((aligned(16))) bf16_t As[GM * LDT];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[GN * LDT];
     __shared__ int s_pair[GM];
-    static_assert(MODE == 1 || GN == 128, "gate and up rows come as 64 and 64");
+    static_assert(MODE != 0 || GN == 128, "gate and up rows come as 64 and 64");
     const int t = blockIdx.x % max_tiles, tn = blockIdx.x / max_tiles;     // neighbouring workgroups share a column tile
     if (t >= work[0]) return;
     const int32_t *tile = work + 1 + 3 * t, *order = work + 1 + 3 * max_tiles;
@@ -135,7 +137,8 @@ grouped_tiles_kernel(const bf16_t *__restrict__ x, int ldx, const int32_t *__res
             const int row = chunk / (GK / 8), k = k0 + (chunk % (GK / 8)) * 8;
             const int pair = s_pair[row];
             // MODE 0 reads the scaled rows, which lie in slot order; MODE 1 the activations, which lie in pair order
-            ra[c] = (pair >= 0 && k < k_end) ? *(const bf16x8_t *)(x + (size_t)(MODE == 0 ? first + row : pair) * ldx + k) : zero8();
+            const size_t from = MODE == 0 ? first + row : (MODE == 2 ? (pair < 0 ? 0 : pair / top) : pair);
+            ra[c] = (pair >= 0 && k < k_end) ? *(const bf16x8_t *)(x + from * ldx + k) : zero8();
         }
 #pragma unroll
         for (int c = 0; c < kB; c++) {
@@ -196,6 +199,13 @@ grouped_tiles_kernel(const bf16_t *__restrict__ x, int ldx, const int32_t *__res
                 u = fminf(fmaxf(u, -limit), limit);
             }
             act[(size_t)pair * N + n] = (bf16_t)(g / (1.0f + expf(-alpha * g)) * (u + up_offset));
+        } else if (MODE == 2) {
+#pragma unroll
+            for (int j = 0; j < CJ; j++) {
+                const int n = n0 + wn * (GN / 2) + j * 32 + l32;
+                const float a = fmaxf(acc[i][j][v], 0.f);
+                if (n < N) act[(size_t)pair * N + n] = (bf16_t)(a * a);
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < CJ; j++) {
@@ -270,7 +280,7 @@ extern "C" int fllm_experts_grouped(const void *h, int ldh, const int32_t *ids, 
     hipLaunchKernelGGL((grouped_tiles_kernel<MODE, ROWS, COLS>),                                                                           \
                        dim3((unsigned)(max_tiles * (MODE == 0 ? up_tiles : down_tiles)), MODE == 0 ? 1 : slices), dim3(kThreads), 0,        \
                        stream, (const bf16_t *)(X), LDX, work, (int)max_tiles, (const bf16_t *)(W), NN, KK, (bf16_t *)act, down_out, limit, \
-                       alpha, up_offset, MODE == 0 ? KK : k_per_down, (size_t)pairs * N)
+                       alpha, up_offset, MODE == 0 ? KK : k_per_down, (size_t)pairs * N, top)
     if (GM == 128) FLLM_GROUPED(0, 128, 128, xs, K, w_gate_up, inter, K);
     else FLLM_GROUPED(0, 64, 128, xs, K, w_gate_up, inter, K);
     if (GM == 128 && GN_DOWN == 128) FLLM_GROUPED(1, 128, 128, act, inter, w_down, N, inter);
@@ -283,4 +293,47 @@ extern "C" int fllm_experts_grouped(const void *h, int ldh, const int32_t *ids, 
         hipLaunchKernelGGL(sum_planes_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, planes, out, count, slices);
     }
     return fllm_check_launch("experts_grouped");
+}
+
+// The same for experts without a gate: act = relu(W_up[e] h)^2 on the rows as they are, then the down product.  w_up
+// [E][inter][K]; no scaled copies of the rows are needed.  0: launched, negative: error, 1: shape declined.
+extern "C" int fllm_experts_grouped_ungated(const void *h, int ldh, const int32_t *ids, int rows, int top, const void *w_up,
+                                            const void *w_down, int E, int inter, int K, int N, void *act, float *out, int32_t *work,
+                                            float *planes, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && top > 0 && E > 0 && inter > 0 && K > 0 && N > 0 && ldh >= K, "experts_grouped_ungated: bad sizes");
+    FLLM_REQUIRE(h && ids && w_up && w_down && act && out && work, "experts_grouped_ungated: operands missing");
+    if (!fllm_fast_kernels_enabled()) return 1;
+    if (K % 8 != 0 || inter % 8 != 0 || ldh % 8 != 0 || E > 4096) return 1;
+    if ((((uintptr_t)h | (uintptr_t)w_up | (uintptr_t)w_down | (uintptr_t)act) & 15) != 0) return 1;
+    const long pairs = (long)rows * top;
+    if (pairs == 0) return 0;
+    const int GM = pairs / E >= 96 ? 128 : 64;
+    const long max_tiles = (pairs + GM - 1) / GM + E;
+    const int GN_UP = max_tiles * ((inter + 127) / 128) < 256 ? 64 : 128;
+    const int GN_DOWN = max_tiles * ((N + 127) / 128) < 256 ? 64 : 128;
+    const int slices = GN_DOWN == 64 ? down_slices(pairs, E, N, inter) : 1;
+    FLLM_REQUIRE(slices == 1 || planes != nullptr, "experts_grouped_ungated: the planes of a down product cut along K are missing");
+    const int k_per_down = slices > 1 ? ((inter + slices - 1) / slices + GK - 1) / GK * GK : inter;
+    const long up_tiles = (inter + GN_UP - 1) / GN_UP, down_tiles = (N + GN_DOWN - 1) / GN_DOWN;
+    if (pairs > (1L << 24) || max_tiles * up_tiles > 0x7fffffffL || max_tiles * down_tiles > 0x7fffffffL) return 1;
+    hipLaunchKernelGGL(group_pairs_kernel, dim3(1), dim3(1024), (size_t)3 * E * sizeof(int), stream, ids, (int)pairs, E, (int)max_tiles, GM, work);
+    float *down_out = slices > 1 ? planes : out;
+#define FLLM_UNGATED(MODE, ROWS, COLS, X, LDX, W, NN, KK, TILES, SLICES, KPER)                                                          \
+    hipLaunchKernelGGL((grouped_tiles_kernel<MODE, ROWS, COLS>), dim3((unsigned)(max_tiles * (TILES)), SLICES), dim3(kThreads), 0, stream, \
+                       (const bf16_t *)(X), LDX, work, (int)max_tiles, (const bf16_t *)(W), NN, KK, (bf16_t *)act, down_out, 0.f, 0.f, 0.f, \
+                       KPER, (size_t)pairs * N, top)
+    if (GM == 128 && GN_UP == 128) FLLM_UNGATED(2, 128, 128, h, ldh, w_up, inter, K, up_tiles, 1, K);
+    else if (GM == 128) FLLM_UNGATED(2, 128, 64, h, ldh, w_up, inter, K, up_tiles, 1, K);
+    else if (GN_UP == 128) FLLM_UNGATED(2, 64, 128, h, ldh, w_up, inter, K, up_tiles, 1, K);
+    else FLLM_UNGATED(2, 64, 64, h, ldh, w_up, inter, K, up_tiles, 1, K);
+    if (GM == 128 && GN_DOWN == 128) FLLM_UNGATED(1, 128, 128, act, inter, w_down, N, inter, down_tiles, slices, k_per_down);
+    else if (GM == 128) FLLM_UNGATED(1, 128, 64, act, inter, w_down, N, inter, down_tiles, slices, k_per_down);
+    else if (GN_DOWN == 128) FLLM_UNGATED(1, 64, 128, act, inter, w_down, N, inter, down_tiles, slices, k_per_down);
+    else FLLM_UNGATED(1, 64, 64, act, inter, w_down, N, inter, down_tiles, slices, k_per_down);
+#undef FLLM_UNGATED
+    if (slices > 1) {
+        const size_t count = (size_t)pairs * N;
+        hipLaunchKernelGGL(sum_planes_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, planes, out, count, slices);
+    }
+    return fllm_check_launch("experts_grouped_ungated");
 }

@@ -141,10 +141,10 @@ def load_library(build_if_missing: bool = True):
         "fllm_pool_blocks": [c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int,
                              c_int, c_int, c_void],
         "fllm_pooled_window_attention": [c_void, c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void,
-                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void],
+                                         c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_sigmoid_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int, c_int,
                                    c_int, c_int, c_int, c_int, c_float, c_float, c_void, c_void, c_void, c_float, c_int, c_int, c_int,
-                                   c_void],
+                                   c_int, c_void],
         "fllm_rotate_scale": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int,
                               c_void],
         "fllm_group_norm_gate": [c_void, c_int, c_float, c_int, c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void],
@@ -153,6 +153,8 @@ def load_library(build_if_missing: bool = True):
         "fllm_relu_squared": [c_void, c_void, c_size, c_int, c_void],
         "fllm_route_grouped": [c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void, c_float, c_int,
                                c_void],
+        "fllm_experts_grouped_ungated": [c_void, c_int, c_void, c_int, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void,
+                                         c_void, c_void, c_void],
         "fllm_experts_up": [c_void, c_int, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_void, c_int, c_void],
     }
     for name, args in sig.items():
@@ -1243,7 +1245,7 @@ class Ops:
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(pool_k), _ptr(pool_v), _ptr(tables), tables.shape[1], _ptr(row_pos),
             _ptr(row_seg), _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, k_dim, v_dim, page_size,
             float(scale), int(window), int(pool), key_chunk,
-            _DTYPE_CODE[q.dtype], self._stream()))
+            _DTYPE_CODE[q.dtype], int(max_context), self._stream()))
         return out
 
     def sigmoid_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, tables: torch.Tensor, row_pos: torch.Tensor,
@@ -1260,7 +1262,7 @@ class Ops:
         self._check(self.lib.fllm_sigmoid_attention(
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg), _ptr(seg_start),
             seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, k_dim, v_dim, page_size, float(scale), float(softcap), _ptr(r1), _ptr(r2), _ptr(pb), float(temp_coef),
-            int(temp_every), key_chunk, _DTYPE_CODE[q.dtype], self._stream()))
+            int(temp_every), key_chunk, _DTYPE_CODE[q.dtype], int(max_context), self._stream()))
         return out
 
     def rotate_scale(self, qkv: torch.Tensor, out: torch.Tensor, row_pos: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, heads: int,
@@ -1359,6 +1361,33 @@ class Ops:
         self._check(self.lib.fllm_experts_up(_ptr(h), h.stride(0) if rows > 1 else K, _ptr(ids), rows, top, _ptr(w_up), E, inter, K,
                                              _ptr(act), _DTYPE_CODE[h.dtype], self._stream()))
         return act
+
+    def experts_grouped_ungated(self, h: torch.Tensor, ids: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, out: torch.Tensor) -> bool:
+        """`experts_up` and `experts_down` in one call on the matrix cores (bfloat16, steps with enough pairs an expert): the
+        pairs are grouped by expert on the device.  out float32 [rows * top, width].  False: not taken, nothing was written."""
+        rows, K = h.shape
+        top = ids.shape[1]
+        E, inter = w_up.shape[0], w_up.shape[1]
+        if h.dtype != torch.bfloat16 or not h.is_cuda:
+            return False
+        if rows < self.GROUPED_EXPERTS_ROWS and rows * top < self.GROUPED_EXPERTS_SHARE * E:
+            return False
+        N = w_down.shape[1]
+        _need(h.dim() == 2 and h.stride(1) == 1, "h must be a row-major matrix")
+        _dense(w_up, "w_up", h.dtype, (E, inter, K))
+        _dense(w_down, "w_down", h.dtype, (E, N, inter))
+        _dense(ids, "ids", torch.int32, (rows, top))
+        _dense(out, "out", torch.float32, (rows * top, N))
+        act = torch.empty((rows * top, inter), dtype=h.dtype, device=h.device)
+        work = torch.empty((int(self.lib.fllm_experts_grouped_work_ints(rows * top, E)),), dtype=torch.int32, device=h.device)
+        need = int(self.lib.fllm_experts_grouped_plane_floats(rows * top, E, N, inter))
+        planes = torch.empty((need,), dtype=torch.float32, device=h.device) if need else None
+        code = self.lib.fllm_experts_grouped_ungated(_ptr(h), h.stride(0), _ptr(ids), rows, top, _ptr(w_up), _ptr(w_down), E, inter, K, N,
+                                                     _ptr(act), _ptr(out), _ptr(work), _ptr(planes), self._stream())
+        if code == 1:
+            return False
+        self._check(code)
+        return True
 
     def measured_ceilings(self, read_bytes: int = 4 << 30, repeats: int = 5) -> dict:
         """What the device delivers to kernels that do nothing else: GB/s of a kernel that only reads a buffer much larger

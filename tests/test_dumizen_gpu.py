@@ -102,7 +102,7 @@ def test_queries_and_keys_normed_rotated_and_stored(ops, ref, H, G, d, dv, rope,
     qkv = torch.randn(sc.rows, width, generator=g).to(dtype).float()
     qw = 1 + 0.4 * torch.rand(H * d if mode == 2 else d, generator=g)
     kw = 1 + 0.4 * torch.rand(G * d if mode == 2 else d, generator=g)
-    cos, sin = torch.rand(300, rope // 2, generator=g) * 2 - 1, torch.rand(300, rope // 2, generator=g) * 2 - 1
+    cos, sin = torch.rand(400, rope // 2, generator=g) * 2 - 1, torch.rand(400, rope // 2, generator=g) * 2 - 1
     results = []
     for o, dev, kind in ((ref, "cpu", torch.float64), (ops, DEV, dtype)):
         t = sc.to(dev, kind)
@@ -334,6 +334,27 @@ def test_experts_without_a_gate(ops, ref, rows, width, inter, experts, top, dtyp
     ops.experts_up(h.to(DEV), ids.to(DEV), w_up.to(DEV), got)
     close(got, want, *((1e-5, 1e-5) if dtype == torch.float32 else (BF16_EPS, 1e-3)), "activations")
     assert (want == 0).float().mean() > 0.2          # the negative half is cut off
+
+
+@pytest.mark.parametrize("spread", ["random", "one expert"])
+@pytest.mark.parametrize("rows,width,inter,experts,top", [(17, 64, 24, 6, 2), (70, 136, 40, 4, 2), (300, 320, 96, 8, 4), (1000, 256, 136, 16, 3),
+                                                          (4, 128, 64, 2, 2)])
+def test_experts_without_a_gate_grouped_on_the_matrix_cores(ops, ref, rows, width, inter, experts, top, spread):
+    g = gen(rows + inter)
+    h = torch.randn(rows, width, generator=g).to(torch.bfloat16)
+    w_up = (torch.randn(experts, inter, width, generator=g) * 2 * width ** -0.5).to(torch.bfloat16)
+    w_down = (torch.randn(experts, width, inter, generator=g) * inter ** -0.5).to(torch.bfloat16)
+    if spread == "random":
+        ids = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(rows)]).to(torch.int32)
+    else:
+        ids = torch.arange(top, dtype=torch.int32).repeat(rows, 1)
+    act = torch.empty(rows * top, inter, dtype=torch.float64)
+    ref.experts_up(h.double(), ids, w_up.double(), act)
+    want = torch.empty(rows * top, width, dtype=torch.float64)
+    ref.experts_down(act.to(torch.bfloat16).double(), ids, w_down.double(), want)
+    got = torch.full((rows * top, width), float("nan"), device=DEV)
+    assert ops.experts_grouped_ungated(h.to(DEV), ids.to(DEV), w_up.to(DEV), w_down.to(DEV), got)
+    close(got, want, 2 * BF16_EPS, 2e-2 * want.abs().max().item(), "grouped experts")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
