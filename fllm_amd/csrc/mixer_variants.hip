@@ -125,15 +125,24 @@ pool_blocks_kernel(const T *__restrict__ k_pages, const T *__restrict__ v_pages,
     const int first = pos - pool + 1;
     const size_t dst = (((size_t)tbl[pos / page_size] * kv_heads + kvh) * slots + (pos % page_size) / pool);
     for (int c = threadIdx.x; c < k_dim + v_dim; c += kBlock) {
+        const bool is_key = c < k_dim;
+        const int cv = c - k_dim;
         float sum = 0.f;
-#pragma unroll 8      // eight loads on their way at once
-        for (int t = 0; t < pool; t++) {
-            const int key = first + t, page = tbl[key / page_size], off = key % page_size;
-            sum += c < k_dim ? to_f32<T>(k_pages[key_at(page, kv_heads, kvh, page_size, k_dim, off, c, key_chunk)])
-                             : to_f32<T>(v_pages[(((size_t)page * kv_heads + kvh) * v_dim + (c - k_dim)) * page_size + off]);
+        for (int t0 = 0; t0 < pool; t0 += 8) {      // eight loads on their way at once, added in position order
+            float vals[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int key = first + (t0 + j < pool ? t0 + j : pool - 1), page = tbl[key / page_size], off = key % page_size;
+                const size_t at = is_key ? key_at(page, kv_heads, kvh, page_size, k_dim, off, c, key_chunk)
+                                         : (((size_t)page * kv_heads + kvh) * v_dim + cv) * page_size + off;
+                vals[j] = to_f32<T>((is_key ? k_pages : v_pages)[at]);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (t0 + j < pool) sum += vals[j];
         }
-        if (c < k_dim) pool_k[dst * k_dim + c] = sum / (float)pool;
-        else pool_v[dst * v_dim + (c - k_dim)] = sum / (float)pool;
+        if (is_key) pool_k[dst * k_dim + c] = sum / (float)pool;
+        else pool_v[dst * v_dim + cv] = sum / (float)pool;
     }
 }
 

@@ -43,6 +43,12 @@ struct TileParams {
     float *parts;                             // [tile][split][16 * DV sums, 16 maxima, 16 denominators] for the merge kernel
 };
 
+// The hardware's exponential, logarithm and reciprocal (a unit or two in the last place of a float32): these kernels serve the
+// bfloat16 path alone, whose operands are rounded to eight bits.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0.6931471805599453f; }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
 __device__ __forceinline__ void split_bf16(const float (&x)[8], bf16x8_t &hi, bf16x8_t &lo) {
 #pragma unroll
     for (int e = 0; e < 8; e++) {
@@ -125,6 +131,7 @@ mixer_tile_kernel(const TileParams p) {
         a1 = p.r1[my_head], a2 = p.r2[my_head], bias = p.pb[my_head];
     }
     const float sc = p.scale * temp;
+    const float two_over_cap = VARIANT == 1 ? 2.0f / p.softcap : 0.f;
     int turn = 0;      // blocks are dealt to the waves in turn, over both kinds of keys
 
     // one block of 32 keys: scores in s[2], then weights, then the products with the values
@@ -142,13 +149,13 @@ mixer_tile_kernel(const TileParams p) {
             m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, kWave));
             m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave));
             const float m_new = fmaxf(m_run, m_blk);
-            const float alpha = m_run == -INFINITY ? 0.f : expf(m_run - m_new);
+            const float alpha = m_run == -INFINITY ? 0.f : fast_exp(m_run - m_new);
             float sum = 0.f;
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const float pv = s[j][i] == -INFINITY ? 0.f : expf(s[j][i] - m_new);
+                    const float pv = s[j][i] == -INFINITY ? 0.f : fast_exp(s[j][i] - m_new);
                     pvals[j * 4 + i] = pv;
                     sum += pv;
                 }
@@ -162,9 +169,11 @@ mixer_tile_kernel(const TileParams p) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int slot = g * 8 + j * 4 + i;
+                    // cap * tanh(x / cap) = cap - 2 cap / (exp(2 x / cap) + 1): an overflowing exponential gives cap, none -cap
                     float x = s[j][i] * sc;
-                    x = p.softcap * tanhf(x / p.softcap) - a1 * log1pf(a2 * distance(slot)) + bias;
-                    pvals[j * 4 + i] = visible(slot) ? 1.0f / (1.0f + expf(-x)) : 0.f;
+                    x = p.softcap - 2.0f * p.softcap * fast_rcp(fast_exp(x * two_over_cap) + 1.0f);
+                    x = x - a1 * fast_log(fmaf(a2, distance(slot), 1.0f)) + bias;
+                    pvals[j * 4 + i] = visible(slot) ? fast_rcp(1.0f + fast_exp(-x)) : 0.f;
                 }
         }
         bf16x8_t p_hi, p_lo;
