@@ -158,9 +158,10 @@ def _attention(m, where: str, kind: str) -> AttentionSizes:
         softcap = _need(m, "softcap", float, where)
         if not softcap > 0.0:
             raise ConfigError(f"{where}softcap must be positive, is {softcap}")
-        temp = _need(m, "q_temp", dict, where)
-        extra.update(softcap=softcap, temp_coef=_need(temp, "coef", float, where + "q_temp."),
-                     temp_every=_positive(temp, "every", where + "q_temp."))
+        extra.update(softcap=softcap)
+        if m.get("q_temp") is not None:       # absent: the queries keep their temperature of 1
+            temp = _need(m, "q_temp", dict, where)
+            extra.update(temp_coef=_need(temp, "coef", float, where + "q_temp."), temp_every=_positive(temp, "every", where + "q_temp."))
     elif vdim != dim:          # the left mixer of a pair: its keys are its values
         raise ConfigError(f"{where}vdim {vdim} must equal dim {dim}: the values of this mixer are its keys")
     rot = None if kind == "attention_2" else _rotation(m, where, dim)

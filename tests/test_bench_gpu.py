@@ -101,6 +101,26 @@ def test_the_line_of_the_design_with_routed_layers():
 
 
 @pytest.mark.gpu
+def test_the_line_of_the_design_with_pooled_windows():
+    """`--design dumizen`: sigmoid, windowed and paired layers, all routed, beside Purivik and Llama at equal sizes."""
+    done = run_bench("--design", "dumizen", "--design-size", "small", "--layers", "4", "--steps", "6", "--warmup", "2",
+                     "--repeats", "1")
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = done.stdout.strip().splitlines()
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    assert line["layer_runs"] == 6 and line["sizes"]["layers"] == 4 and line["dtype"] == "bf16"
+    for model in ("dumizen", "purivik", "llama"):
+        got = line[model]
+        assert set(got) >= {"decode_b1", "decode_b8", "decode_b64", "prefill", "kernels"}
+        assert got["decode_b64"]["tokens_per_s"] > got["decode_b1"]["tokens_per_s"] > 0
+    # prompts and decode steps run the tile kernel of the two new attentions and the experts grouped on the matrix cores
+    prefill, decode = " ".join(line["dumizen"]["kernels"]["prefill_us"]), " ".join(line["dumizen"]["kernels"]["decode_b8_us"])
+    assert "mixer_tile_kernel" in prefill and "grouped_tiles_kernel<2" in prefill and "sigmoid_attention_kernel" not in prefill
+    assert "pooled_window_attention_kernel" not in prefill and "mixer_tile_kernel" in decode
+
+
+@pytest.mark.gpu
 def test_the_smoke_run_of_the_entry_file():
     """`__graft_entry__.smoke()` in a process of its own, as it is run: a few tokens of a tiny random model on the
     device against the plain implementation."""
