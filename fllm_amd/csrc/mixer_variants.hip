@@ -146,6 +146,59 @@ pool_blocks_kernel(const T *__restrict__ k_pages, const T *__restrict__ v_pages,
     }
 }
 
+// The same for bfloat16 pages with keys in chunks of 8, blocks of a multiple of 8 positions and pages of a multiple of 8
+// tokens: every load takes 16 bytes (8 lanes of a key, or 8 tokens of a value lane), a thread sums eight positions in
+// order, and the eights are added in order through LDS: two rounds of loads a block instead of one a position.
+__global__ void __launch_bounds__(kBlock)
+pool_blocks_vec_kernel(const bf16_t *__restrict__ k_pages, const bf16_t *__restrict__ v_pages, float *__restrict__ pool_k,
+                       float *__restrict__ pool_v, const int32_t *__restrict__ tables, int table_stride,
+                       const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seg, int kv_heads, int k_dim, int v_dim,
+                       int page_size, int pool, int slots) {
+    extern __shared__ float part[];      // [pool / 8][k_dim + v_dim]
+    const int r = blockIdx.x, kvh = blockIdx.y;
+    const int seg = row_seg[r];
+    if (seg < 0) return;
+    const int pos = row_pos[r];
+    if ((pos + 1) % pool != 0) return;
+    const int32_t *tbl = tables + (size_t)seg * table_stride;
+    const int first = pos - pool + 1, eights = pool / 8, width = k_dim + v_dim;
+    const size_t dst = (((size_t)tbl[pos / page_size] * kv_heads + kvh) * slots + (pos % page_size) / pool);
+    // keys: an item is (eight positions, one chunk of 8 lanes)
+    for (int item = threadIdx.x; item < eights * (k_dim / 8); item += kBlock) {
+        const int tg = item / (k_dim / 8), ch = item - tg * (k_dim / 8);
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        bf16x8_t got[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int key = first + tg * 8 + j;
+            got[j] = *(const bf16x8_t *)(k_pages + key_offset(tbl[key / page_size], kv_heads, kvh, page_size, k_dim, key % page_size, ch * 8));
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] += (float)got[j][e];
+#pragma unroll
+        for (int e = 0; e < 8; e++) part[tg * width + ch * 8 + e] = acc[e];
+    }
+    // values: an item is (eight positions, one lane); the eight lie side by side in one page
+    for (int item = threadIdx.x; item < eights * v_dim; item += kBlock) {
+        const int tg = item / v_dim, c = item - tg * v_dim;
+        const int key = first + tg * 8;
+        const bf16x8_t got = *(const bf16x8_t *)(v_pages + (((size_t)tbl[key / page_size] * kv_heads + kvh) * v_dim + c) * page_size + key % page_size);
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc += (float)got[e];
+        part[tg * width + k_dim + c] = acc;
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < width; c += kBlock) {
+        float sum = 0.f;
+        for (int tg = 0; tg < eights; tg++) sum += part[tg * width + c];
+        if (c < k_dim) pool_k[dst * k_dim + c] = sum / (float)pool;
+        else pool_v[dst * v_dim + (c - k_dim)] = sum / (float)pool;
+    }
+}
+
 // ---- what a thread's key contributes ---------------------------------------------------------------------------------------
 template <typename T>
 __device__ __forceinline__ float key_dot(const float *__restrict__ qs, const T *__restrict__ kr, int head_dim, size_t chunk_step, int key_chunk) {
@@ -493,6 +546,11 @@ extern "C" int fllm_pool_blocks(const void *k_pages, const void *v_pages, float 
         hipLaunchKernelGGL(pool_blocks_kernel<float>, dim3(rows, kv_heads), dim3(kBlock), 0, stream, (const float *)k_pages,
                            (const float *)v_pages, pool_k, pool_v, tables, table_stride, row_pos, row_seg, kv_heads, k_dim, v_dim,
                            page_size, key_chunk, pool, slots);
+    else if (dtype == FLLM_BF16 && key_chunk == 8 && pool % 8 == 0 && page_size % 8 == 0 &&
+             (size_t)(pool / 8) * (k_dim + v_dim) * sizeof(float) <= 48 * 1024)
+        hipLaunchKernelGGL(pool_blocks_vec_kernel, dim3(rows, kv_heads), dim3(kBlock), (size_t)(pool / 8) * (k_dim + v_dim) * sizeof(float), stream,
+                           (const bf16_t *)k_pages, (const bf16_t *)v_pages, pool_k, pool_v, tables, table_stride, row_pos, row_seg, kv_heads,
+                           k_dim, v_dim, page_size, pool, slots);
     else if (dtype == FLLM_BF16)
         hipLaunchKernelGGL(pool_blocks_kernel<bf16_t>, dim3(rows, kv_heads), dim3(kBlock), 0, stream, (const bf16_t *)k_pages,
                            (const bf16_t *)v_pages, pool_k, pool_v, tables, table_stride, row_pos, row_seg, kv_heads, k_dim, v_dim,
