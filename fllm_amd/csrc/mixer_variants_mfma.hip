@@ -2,7 +2,7 @@
 //
 // A workgroup of four waves takes one tile of up to 16 queries: 16 rows of one request and one head (prompt portions), or
 // the heads of one key/value head of one row (steps of single rows).  The waves deal the tile's keys among themselves in
-// blocks of 32 and meet in LDS at the end.  Nothing is staged: every operand is a 16-byte load straight from the pages, which
+// pairs of blocks of 32 and meet in LDS at the end.  Nothing is staged: every operand is a 16-byte load straight from the pages, which
 // hold 8 lanes of a key side by side and a value lane's tokens side by side.
 //
 //   S^T = K Q^T   v_mfma_f32_16x16x32_bf16, A = 16 keys x 32 lanes, B = Q^T: the result leaves lane l with its own query
@@ -232,38 +232,52 @@ mixer_tile_kernel(const TileParams p) {
                 });
         }
     }
-    // ---- the tokens: from the first one that the tile's first row sees, in blocks of 32 positions
+    // ---- the tokens: from the first one that the tile's first row sees, two blocks of 32 positions a turn.  All operands of a
+    // turn are asked for before the first product, so that the second block's loads and both blocks' values travel while the
+    // first block's scores are weighed.  Keys behind the tile's last row are read from an address that exists and masked.
     {
         const int first = VARIANT == 0 ? (pos_min - p.window + 1 > 0 ? pos_min - p.window + 1 : 0) : 0;
-        for (int base = first & ~31; base <= pos_max; base += 32, turn++) {
+        for (int base0 = first & ~63; base0 <= pos_max; base0 += 64, turn++) {
             if ((turn & (kWavesM - 1)) != wave || (turn / kWavesM) % p.splits != (int)blockIdx.z) continue;
-            f32x4_t s[2];
+            bf16x8_t ka[2][2][KD], va[2][VT];
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                s[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
-                int key = base + (qi >> 2) * 8 + j * 4 + (qi & 3);
-                key = key <= pos_max ? key : pos_max;      // keys behind the tile's last row: any address that exists
-                const bf16_t *kr = p.k_pages + key_offset(tbl[key / ps], p.kv_heads, kvh, ps, D, key % ps, g * 8);
+            for (int half = 0; half < 2; half++) {
+                const int base = base0 + half * 32;
 #pragma unroll
-                for (int kk = 0; kk < KD; kk++) {
-                    const bf16x8_t a = *(const bf16x8_t *)(kr + (size_t)kk * 4 * ps * 8);      // 32 lanes on: four chunks of 8
-                    s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[kk], s[j], 0, 0, 0);
+                for (int j = 0; j < 2; j++) {
+                    int key = base + (qi >> 2) * 8 + j * 4 + (qi & 3);
+                    key = key <= pos_max ? key : pos_max;
+                    const bf16_t *kr = p.k_pages + key_offset(tbl[key / ps], p.kv_heads, kvh, ps, D, key % ps, g * 8);
+#pragma unroll
+                    for (int kk = 0; kk < KD; kk++) ka[half][j][kk] = *(const bf16x8_t *)(kr + (size_t)kk * 4 * ps * 8);      // 32 lanes on: four chunks of 8
                 }
-            }
-            weigh_and_add(
-                s, [&](int slot) { const int key = base + slot; return valid && key <= my_pos && key >= lo_q; },
-                [&](int slot) { const int dist = my_pos - (base + slot); return (float)(dist > 0 ? dist : 0); },
-                [&](const bf16x8_t &p_hi, const bf16x8_t &p_lo) {
-                    int key = base + g * 8;                  // eight tokens side by side in one page (pages hold multiples of 16)
-                    key = key <= pos_max ? key : pos_max & ~7;
-                    const bf16_t *vr = p.v_pages + (((size_t)tbl[key / ps] * p.kv_heads + kvh) * DV + qi) * ps + key % ps;
+                int key = base + g * 8;                  // eight tokens side by side in one page (pages hold multiples of 16)
+                key = key <= pos_max ? key : pos_max & ~7;
+                const bf16_t *vr = p.v_pages + (((size_t)tbl[key / ps] * p.kv_heads + kvh) * DV + qi) * ps + key % ps;
 #pragma unroll
-                    for (int t = 0; t < VT; t++) {
-                        const bf16x8_t a = *(const bf16x8_t *)(vr + (size_t)t * 16 * ps);
-                        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_hi, o[t], 0, 0, 0);
-                        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, p_lo, o[t], 0, 0, 0);
-                    }
-                });
+                for (int t = 0; t < VT; t++) va[half][t] = *(const bf16x8_t *)(vr + (size_t)t * 16 * ps);
+            }
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                const int base = base0 + half * 32;
+                f32x4_t s[2];
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    s[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kk = 0; kk < KD; kk++) s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[half][j][kk], qf[kk], s[j], 0, 0, 0);
+                }
+                weigh_and_add(
+                    s, [&](int slot) { const int key = base + slot; return valid && key <= my_pos && key >= lo_q; },
+                    [&](int slot) { const int dist = my_pos - (base + slot); return (float)(dist > 0 ? dist : 0); },
+                    [&](const bf16x8_t &p_hi, const bf16x8_t &p_lo) {
+#pragma unroll
+                        for (int t = 0; t < VT; t++) {
+                            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[half][t], p_hi, o[t], 0, 0, 0);
+                            o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[half][t], p_lo, o[t], 0, 0, 0);
+                        }
+                    });
+            }
         }
     }
     // ---- the waves meet

@@ -19,7 +19,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..registry import part_class, register_part
-from .base import INIT_MATRIX, INIT_NORM, Mixer, StateNeed, add_and_prepare
+from .base import INIT_MATRIX, INIT_NORM, Mixer, StateNeed, add_and_prepare, fused_form, take_prepared
 
 
 class LightningAttention(Mixer):
@@ -76,11 +76,28 @@ class LightningAttention(Mixer):
         return StateNeed((self.heads, self.dim, self.v_dim), torch.float32)
 
     def forward(self, ctx, h, residual, binding, branch=None) -> None:
+        qkvg = self.rt.empty((h.shape[0], self.w_qkvg.shape[0]))
+        self.rt.ops.linear(h, self.w_qkvg, qkvg)
+        self.forward_from_projection(ctx, qkvg, residual, binding, branch)
+
+    def project_norm(self, ctx, residual, norm):
+        """Decode-sized steps in bfloat16: the joint product straight from the residual stream, the norm before the mixer
+        folded in, for whoever arranges this mixer and goes on with `forward_from_projection`.  None: not taken."""
         rt, ops = self.rt, self.rt.ops
-        rows = h.shape[0]
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if rt.dtype != torch.bfloat16 or prologue is None or not hasattr(ops, "norm_linear"):
+            return None
+        if fused_form(ops, residual.shape[0], self.hidden, self.w_qkvg) != "resident":
+            return None
+        qkvg = rt.empty((residual.shape[0], self.w_qkvg.shape[0]))
+        ops.norm_linear(residual, prologue[0], prologue[1], self.w_qkvg, qkvg)
+        return qkvg
+
+    def forward_from_projection(self, ctx, qkvg, residual, binding, branch=None) -> None:
+        """From the joint product [q | k | v | gate] of the step's rows to the output projection."""
+        rt, ops = self.rt, self.rt.ops
+        rows = qkvg.shape[0]
         nq, nv = self.heads * self.dim, self.heads * self.v_dim
-        qkvg = rt.empty((rows, 2 * nq + 2 * nv))
-        ops.linear(h, self.w_qkvg, qkvg)
         o = rt.empty((rows, nv), torch.float32)
         operands = qkvg
         if self.position is not None or self.key_scale != 1.0:

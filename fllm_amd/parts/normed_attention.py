@@ -18,7 +18,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..registry import part_class, register_part
-from .base import INIT_BIAS, INIT_MATRIX, INIT_NORM, KVNeed, Mixer, add_and_prepare
+from .base import INIT_BIAS, INIT_MATRIX, INIT_NORM, KVNeed, Mixer, add_and_prepare, fused_form, take_prepared
 
 NORM_MODES = {None: 0, "head": 1, "projection": 2}
 
@@ -109,11 +109,30 @@ class NormedAttention(Mixer):
         return KVNeed(self.kv_heads, self.head_dim, self.v_dim, None, key_chunk=self.key_chunk, pooled=int(self.pool or 0))
 
     def forward(self, ctx, h, residual, binding, branch=None):
+        qkv = self.rt.empty((h.shape[0], self.w_qkv.shape[0]))
+        self.rt.ops.linear(h, self.w_qkv, qkv, bias=self.b_qkv)
+        self._attend(ctx, qkv, residual, binding, branch)
+
+    def forward_from_residual(self, ctx, residual, norm, binding, branch=None) -> bool:
+        """Decode-sized steps in bfloat16: the norm before the mixer and the joint product are one kernel that reads the
+        residual stream.  False: not taken, the block runs the norm and `forward`."""
         rt, ops = self.rt, self.rt.ops
-        rows = h.shape[0]
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if rt.dtype != torch.bfloat16 or prologue is None or not hasattr(ops, "norm_linear"):
+            return False
+        if fused_form(ops, residual.shape[0], self.hidden, self.w_qkv) != "resident":
+            return False
+        take_prepared(ctx, norm, residual)          # whatever was prepared for this norm is not used here
+        qkv = rt.empty((residual.shape[0], self.w_qkv.shape[0]))
+        ops.norm_linear(residual, prologue[0], prologue[1], self.w_qkv, qkv, bias=self.b_qkv)
+        self._attend(ctx, qkv, residual, binding, branch)
+        return True
+
+    def _attend(self, ctx, qkv, residual, binding, branch=None):
+        """From the joint product [q | k | v | gate] of the step's rows to the output projection."""
+        rt, ops = self.rt, self.rt.ops
+        rows = qkv.shape[0]
         nh, nkv, d, dv = self.heads, self.kv_heads, self.head_dim, self.v_dim
-        qkv = rt.empty((rows, self.w_qkv.shape[0]))
-        ops.linear(h, self.w_qkv, qkv, bias=self.b_qkv)
         tables = ctx.tables[binding.group]
         if self.position is not None:
             cos, sin, dims = self.position.cos, self.position.sin, self.position.dims

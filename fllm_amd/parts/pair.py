@@ -12,7 +12,7 @@ from types import SimpleNamespace
 import torch
 
 from ..registry import part_class, register_part
-from .base import Mixer, StateNeed
+from .base import Mixer, StateNeed, fused_form
 
 
 class MixerPair(Mixer):
@@ -85,13 +85,41 @@ class MixerPair(Mixer):
                                pool_v=getattr(binding, "pool_v", None) if keeps else None)
 
     def forward(self, ctx, h, residual, binding, branch=None) -> None:
-        rt, ops = self.rt, self.rt.ops
-        rows = h.shape[0]
+        rt = self.rt
         outs = []
         for side, part in self.sides:
-            out = rt.empty((rows, self.size), torch.float32)
+            out = rt.empty((h.shape[0], self.size), torch.float32)
             part.forward(ctx, h, None, self._binding(binding, side, part), branch=out)
             outs.append(out)
+        self._sum(outs, residual, branch)
+
+    def forward_from_residual(self, ctx, residual, norm, binding, branch=None) -> bool:
+        """Decode-sized steps: each side reads the residual stream through the norm in the kernel of its own first product,
+        where both sides have such a form (the norm's few operations are done twice, its launch and its pass not at all).
+        False: not taken."""
+        joint = [getattr(part, "forward_from_residual", None) or getattr(part, "project_norm", None) for _, part in self.sides]
+        if any(j is None for j in joint) or self.rt.dtype != torch.bfloat16:
+            return False
+        # both sides must take it: a side that declines after the other has stored its keys would run that side twice
+        rows = residual.shape[0]
+        if any(fused_form(self.rt.ops, rows, self.size, getattr(part, "w_qkv", getattr(part, "w_qkvg", None))) != "resident"
+               for _, part in self.sides) or getattr(norm, "fused_prologue", lambda: None)() is None:
+            return False
+        outs = []
+        for side, part in self.sides:
+            out = self.rt.empty((rows, self.size), torch.float32)
+            inner = self._binding(binding, side, part)
+            if hasattr(part, "forward_from_residual"):
+                if not part.forward_from_residual(ctx, residual, norm, inner, branch=out):
+                    raise RuntimeError(f"the {side} mixer of a pair declined a step its sizes fit")
+            else:
+                part.forward_from_projection(ctx, part.project_norm(ctx, residual, norm), None, inner, branch=out)
+            outs.append(out)
+        self._sum(outs, residual, branch)
+        return True
+
+    def _sum(self, outs, residual, branch) -> None:
+        ops = self.rt.ops
         if branch is not None:
             ops.weighted_sum(branch, outs[0], self.scales[0], outs[1], self.scales[1])
         else:
