@@ -548,6 +548,33 @@ def test_the_residual_stream_after_every_layer_run(models):
         assert np.abs(got - ref_x).max() <= 1e-5 * np.abs(ref_x).max()
 
 
+def test_decode_steps_take_the_fused_forms_and_prompts_the_tile_kernels(models, monkeypatch):
+    """D in bfloat16 (4 layer runs: sigmoid, windowed twice, a pair): a decode step reads the stream through a layer's first
+    norm inside the first product of every mixer (a pair's two sides each), so no norm kernel of its own runs but the model's
+    last; a prompt runs the norm, and its experts go to the matrix cores grouped by expert."""
+    from fllm_amd.engine import StepEntry
+    from fllm_amd.kernels import Ops
+    folder, cfg, requests, _, _ = models["D", "bfloat16"]
+    runner = make_runner(folder, "bfloat16", 16, 256, use_graphs=False)
+    calls = []
+    for name in ("rmsnorm", "norm_linear", "normed_rope_store", "pool_blocks", "pooled_window_attention", "sigmoid_attention",
+                 "rotate_scale", "linear_attention", "group_norm_gate", "weighted_sum", "route_grouped", "experts_grouped_ungated",
+                 "experts_up", "postnorm_add", "stream_concat"):
+        inner = getattr(Ops, name)
+        monkeypatch.setattr(Ops, name, lambda self, *a, _n=name, _i=inner, **k: (calls.append(_n), _i(self, *a, **k))[1])
+    toks = requests["r0"]
+    runner.step([StepEntry("a", toks[:40], [])])
+    assert calls.count("rmsnorm") == 4 and calls.count("norm_linear") == 0 and calls.count("experts_up") == 0
+    assert calls.count("experts_grouped_ungated") == 4 and calls.count("stream_concat") == 2
+    calls.clear()
+    runner.step([StepEntry("a", toks[40:41], [0])])
+    assert calls.count("norm_linear") == 5 and calls.count("rmsnorm") == 1          # the pair's two sides; the model's last norm
+    assert calls.count("normed_rope_store") == 3 and calls.count("pool_blocks") == 2 and calls.count("pooled_window_attention") == 2
+    assert calls.count("sigmoid_attention") == 1 and calls.count("rotate_scale") == calls.count("linear_attention") == 1
+    assert calls.count("group_norm_gate") == calls.count("weighted_sum") == 1
+    assert calls.count("route_grouped") == 4 and calls.count("postnorm_add") == 12   # a layer run: norm 1b, the picks' sum, norm 2b
+
+
 @pytest.mark.parametrize("name", ["A", "D"])
 def test_greedy_generation_through_the_scheduler(models, name):
     from fllm_amd import Engine, SamplingParams
