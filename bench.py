@@ -268,18 +268,18 @@ def dumizen_config(size, layers):
     """`layers` layers in turn: sigmoid attention over all keys, two of windowed attention (1,024 tokens, blocks of 64 behind
     them) and a pair of attention (its keys as values, a zero sink, an output gate) beside retention (as many heads of the same
     size); routed feed-forwards everywhere: two of eight experts of half the dense width without a gate and a shared one of
-    that width, in two groups of which a token picks inside one (a token multiplies as many weights as the dense gated layer
+    that width, in four groups of which a token picks inside two (a token multiplies as many weights as the dense gated layer
     has); the middle half of the layers runs twice, every pass entered through a matrix of twice the width."""
     heads, kv_heads, dim, ff = size["heads"], size["kv_heads"], size["dim"], size["ff"]
-    scaling = {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}
+    scaling = {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}
     base = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5}
-    sigmoid = dict(base, softcap=50.0, q_temp={"coef": 0.3, "every": 1024})
+    sigmoid = dict(base, softcap=30.0, q_temp={"coef": 0.25, "every": 1024})
     windowed = dict(base, mask={"size": 1024, "pool": 64}, rot={"dims": dim // 2, "base": 500000.0, "scaling": scaling})
-    both = {"left": dict(base, rot={"dims": dim, "base": 1000000.0, "scaling": scaling}), "left_scale": 0.8, "right_scale": 1.1,
+    both = {"left": dict(base, rot={"dims": dim, "base": 1000000.0, "scaling": scaling}), "left_scale": 0.7, "right_scale": 1.2,
             "right": {"heads": heads, "dim": dim, "vdim": dim, "rot": {"dims": dim, "base": 1000000.0},
                       "decay": [1.0 - 2.0 ** -(5 + 5 * h / max(1, heads - 1)) for h in range(heads)]}}
     mlp = {"kind": "moe", "expert": {"ff": ff // DESIGN_TOP}, "shared": {"ff": ff // DESIGN_TOP},
-           "router": {"experts": DESIGN_EXPERTS, "top": DESIGN_TOP, "scale": 2.0, "groups": {"count": 2, "keep": 1}}}
+           "router": {"experts": DESIGN_EXPERTS, "top": DESIGN_TOP, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
     kinds = [("attention_2", sigmoid), ("attention", windowed), ("attention", windowed), ("parallel", both)]
     cfg = {"architecture": "Dumizen", "width": size["width"], "vocab": size["vocab"], "norm": {"eps": 1e-6}, "max_position": 32768,
            "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": mlp} for i in range(layers)]}

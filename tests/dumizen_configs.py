@@ -71,8 +71,8 @@ A = config(64, 96, [
 # key/value heads as heads, a temperature that steps every four positions, a decay of exactly 1
 B = config(96, 120, [
     windowed(3, 3, 32, 32, 5, 1, _rot(32, 10000.0), mlp=(40, 3, 3, 1.0, None, None)),
-    sigmoid(3, 3, 32, 32, 50.0, 0.3, 4, mlp=(40, 4, 2, 2.0, (2, 1), 56)),
-    pair((3, 3, 32, _rot(32, 10000.0), 0.18), (1, 32, 32, (1.0,), None), 1.0, 1.0, mlp=(40, 4, 2, 2.0, (2, 1), 56)),
+    sigmoid(3, 3, 32, 32, 40.0, 0.35, 4, mlp=(40, 4, 2, 1.8, (2, 1), 56)),
+    pair((3, 3, 32, _rot(32, 10000.0), 0.18), (1, 32, 32, (1.0,), None), 1.0, 1.0, mlp=(40, 4, 2, 1.8, (2, 1), 56)),
 ], eps=1e-6)
 # C: sizes that are multiples of nothing (keys lie lane by lane in the pages), blocks of three on pages of sixteen (blocks
 # straddle pages), a window of seven, the whole model looped three times, four groups of one expert
@@ -81,13 +81,13 @@ C = config(68, 77, [
     pair((2, 1, 20, _rot(10, 77.0), 0.25), (3, 10, 6, (0.7, 0.9, 0.999), _rot(10, 20.0)), 0.5, 2.0, mlp=(18, 4, 2, 0.8, (4, 2), 22)),
     sigmoid(3, 1, 12, 20, 3.0, 1.0, 5, scale=0.5),
 ], loop=(0, 3, 3))
-# D: head sizes the matrix-core attention takes on the left (64), long windows, eight experts in two groups, a loop of one
-# layer twice in the middle
+# D: head sizes the matrix-core attention takes on the left (64), long windows with blocks of a page, eight experts in four
+# groups, a loop of one layer twice in the middle
 D = config(128, 160, [
-    sigmoid(4, 2, 64, 64, 20.0, 0.3, 32, scale=0.125, mlp=(48, 8, 3, 2.0, (2, 1), 64)),
-    windowed(8, 2, 64, 32, 40, 8, _rot(32, 20000.0, (4.0, 64, 16.0, 1.0)), scale=0.1, mlp=(48, 8, 3, 2.0, (2, 1), 64)),
-    pair((8, 4, 64, _rot(64, 100000.0, (4.0, 64, 16.0, 1.0)), 0.125), (2, 64, 64, (0.95, 0.999), _rot(64, 100000.0)), 0.8, 1.1,
-         mlp=(48, 8, 3, 2.0, (2, 1), 64)),
+    sigmoid(4, 2, 64, 64, 20.0, 0.25, 32, scale=0.125, mlp=(48, 8, 3, 1.7, (4, 2), 64)),
+    windowed(8, 2, 64, 32, 48, 16, _rot(32, 20000.0, (8.0, 64, 16.0, 1.0)), scale=0.1, mlp=(48, 8, 3, 1.7, (4, 2), 64)),
+    pair((8, 4, 64, _rot(64, 100000.0, (8.0, 64, 16.0, 1.0)), 0.125), (2, 64, 64, (0.95, 0.999), _rot(64, 100000.0)), 0.9, 1.2,
+         mlp=(48, 8, 3, 1.7, (4, 2), 64)),
 ], loop=(1, 2, 2), eps=1e-6)
 CONFIGS = {"A": A, "B": B, "C": C, "D": D}
 PAGE_SIZES = {"A": 8, "B": 16, "C": 16, "D": 16}

@@ -143,7 +143,7 @@ def fill_pools(ref, sc, t, G, d, dv, pool):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,dv,page,window,pool", [(4, 1, 32, 16, 8, 12, 4), (3, 3, 32, 32, 16, 5, 1), (3, 1, 12, 10, 16, 7, 3),
                                                          (8, 2, 64, 32, 16, 40, 8), (2, 1, 128, 300, 32, 33, 16), (12, 2, 128, 128, 16, 100, 8),
-                                                         (6, 2, 96, 32, 32, 40, 8)])
+                                                         (9, 3, 96, 64, 32, 50, 4)])
 def test_windows_with_pooled_blocks_over_pages(ops, ref, H, G, d, dv, page, window, pool, dtype, fast, rows):
     """`fast` False: the plain kernel also where the matrix-core kernel would serve (bfloat16, heads of 32 to 128 lanes in
     steps of 32, pages of multiples of 16); "single": a step of one row a request, whose tiles are the heads of a key/value head."""
@@ -205,7 +205,7 @@ def test_one_key_that_stands_out_at_the_edges(ops, ref, where, held, dtype):
 @pytest.mark.parametrize("fast", [True, False])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,G,d,dv,page", [(4, 2, 16, 24, 8), (3, 3, 32, 32, 16), (3, 1, 12, 20, 16), (4, 2, 64, 64, 16), (2, 1, 96, 300, 32),
-                                           (12, 2, 128, 128, 16), (4, 2, 96, 96, 32)])
+                                           (12, 2, 128, 128, 16), (6, 3, 96, 96, 32)])
 def test_sigmoid_attention_over_pages(ops, ref, H, G, d, dv, page, dtype, fast, rows):
     if dtype == torch.float32 and not fast:
         pytest.skip("float32 has one kernel")
